@@ -1,0 +1,394 @@
+"""``FusedEncoder`` for MI355X: the host side of the single-launch int8 evaluator.
+
+Mirrors the reference class of the same name (brokefish/nn/cuda_impl.py:119-531): built
+from a network, it snapshots the weights into device blobs once, owns its output
+buffers, and ``forward_full(boards, control, rep)`` is one asynchronous kernel launch on
+the current stream returning views of those buffers.
+
+Differences from the reference class, all additive or forced by the parity target:
+
+* the arithmetic reproduced is the reference's PyTorch int8 emulation
+  (brokefish/nn/quant.py:246-305): fp32 activations, LayerNorm affine applied (not folded
+  into the weights), raw weights quantised per 128 output rows, true division;
+* ``forward_full`` takes an optional ``mask`` ([n,32] int64 legal-move words): illegal
+  policy entries come back as -inf and ``best_move`` holds the masked argmax;
+* ``out_dtype=torch.float32`` returns fp32 logits (parity runs); fp16 is the default and
+  the contract the search expects (brokefish/search/cuda_impl.py:242-249).
+
+There is no CPU path: if the HIP library is missing or no GPU is present, construction
+raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Dict, Optional
+
+import numpy as np
+import torch
+
+from . import _build
+
+T, N_POLICY, N_PROMO = 32, 64, 4
+BLOCK_N = 128            # weight-scale block, brokefish/nn/quant.py:82
+Q_MAX_S8, Q_MAX_U8 = 127.0, 255.0   # brokefish/nn/quant.py:237-241
+
+
+class _Shape(C.Structure):
+    _fields_ = [("d_model", C.c_int32), ("n_layers", C.c_int32), ("n_heads", C.c_int32),
+                ("d_ff", C.c_int32), ("n_value", C.c_int32), ("eps", C.c_float)]
+
+
+_TAP_PTRS = ["embed", "qa_qkv", "acc_qkv", "qa_out", "acc_out", "qa_ff1", "acc_ff1",
+             "qa_ff2", "acc_ff2", "resid", "normed"]
+
+
+class _Taps(C.Structure):
+    _fields_ = ([("x_in", C.c_void_p), ("layer_begin", C.c_int32), ("layer_end", C.c_int32)]
+                + [(n, C.c_void_p) for n in _TAP_PTRS])
+
+
+class _Args(C.Structure):
+    _fields_ = [("boards", C.c_void_p), ("control", C.c_void_p), ("rep", C.c_void_p),
+                ("mask", C.c_void_p), ("n", C.c_int64), ("shape", _Shape),
+                ("wstream", C.c_void_p), ("fparams", C.c_void_p),
+                ("policy", C.c_void_p), ("promo", C.c_void_p), ("value", C.c_void_p),
+                ("best_move", C.c_void_p), ("out_fp32", C.c_int32), ("taps", C.POINTER(_Taps))]
+
+
+_lib = None
+
+
+def load_library():
+    """The C-ABI library, loaded once.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        path = _build.HIP_LIB
+        if not os.path.exists(path):
+            raise RuntimeError(
+                f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(hipcc, gfx950). There is no fallback path.")
+        L = C.CDLL(path)
+        L.bf_model_forward.restype = C.c_int
+        L.bf_model_forward.argtypes = [C.POINTER(_Args), C.c_void_p]
+        L.bf_time_kernel_ms.restype = C.c_double
+        L.bf_time_kernel_ms.argtypes = [C.POINTER(_Args), C.c_void_p, C.c_int, C.c_int]
+        L.bf_last_error.restype = C.c_char_p
+        L.bf_wstream_bytes.restype = C.c_size_t
+        L.bf_wstream_bytes.argtypes = [C.POINTER(_Shape)]
+        L.bf_fparams_floats.restype = C.c_size_t
+        L.bf_fparams_floats.argtypes = [C.POINTER(_Shape)]
+        L.bf_int8_q_max.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_double)]
+        _lib = L
+    return _lib
+
+
+def int8_q_max():
+    """(s8, u8) quantisation maxima compiled into the library."""
+    a, b = C.c_double(), C.c_double()
+    load_library().bf_int8_q_max(C.byref(a), C.byref(b))
+    return a.value, b.value
+
+
+# --------------------------------------------------------------------------- #
+# weight packing (host, once per weight generation)
+# --------------------------------------------------------------------------- #
+
+def quantise_weights_int8(w: torch.Tensor):
+    """[N, K] fp32 -> (int8 [N, K], fp32 scale [N // 128]); one scale per 128 output rows
+    over the whole reduction (brokefish/nn/quant.py:263-278)."""
+    n, k = w.shape
+    if n % BLOCK_N:
+        raise ValueError(f"weight {tuple(w.shape)} does not tile into {BLOCK_N} rows")
+    blocks = w.detach().float().cpu().reshape(n // BLOCK_N, BLOCK_N * k)
+    amax = blocks.abs().amax(dim=1, keepdim=True)
+    scale = torch.where(amax > 0, amax / Q_MAX_S8, torch.ones_like(amax))
+    q = torch.round(blocks / scale).clamp(-Q_MAX_S8, Q_MAX_S8).to(torch.int8)
+    return q.reshape(n, k).numpy(), scale.reshape(-1).numpy().astype(np.float32)
+
+
+def _lane_tables():
+    lane = np.arange(64)
+    o, g = lane % 32, lane // 32
+    r = np.arange(16)
+    chan = 8 * (r[None, :] // 4) + 4 * g[:, None] + (r[None, :] % 4)   # [64,16]
+    return o, g, chan
+
+
+def pack_int8_block(wq: np.ndarray, n_tile: int, k0: int) -> np.ndarray:
+    """One 8 KiB block: output tile ``n_tile``, the 256-wide k-chunk starting at ``k0``.
+    Fragment s, lane 32g+o, byte r  <-  wq[32 n_tile + o][k0 + 32 s + ch(r, g)]."""
+    o, _, chan = _lane_tables()
+    rows = (32 * n_tile + o)[None, :, None]                       # [1,64,1]
+    cols = k0 + 32 * np.arange(8)[:, None, None] + chan[None]     # [8,64,16]
+    return np.ascontiguousarray(wq[rows, cols]).view(np.uint8)
+
+
+def pack_head_tile(head: np.ndarray, m: int) -> np.ndarray:
+    """One 32 KiB fp32 head tile: fragment (n, j), lane 32g+o  <-  head[32m+o][32n+8j+4g+0..3]."""
+    d = head.shape[1]
+    o, g, _ = _lane_tables()
+    n = np.arange(d // 32)[:, None, None, None]
+    j = np.arange(4)[None, :, None, None]
+    i = np.arange(4)[None, None, None, :]
+    cols = 32 * n + 8 * j + 4 * g[None, None, :, None] + i         # [NT,4,64,4]
+    rows = (32 * m + o)[None, None, :, None]
+    return np.ascontiguousarray(head[rows, cols], dtype=np.float32)
+
+
+def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_value: int):
+    """state_dict -> (wstream uint8 [bytes], fparams float32 [floats]) in the layouts of
+    include/brokefish_hip.h."""
+    nt, ft, kcf = d // 32, f // 32, f // 256
+    get = lambda k: sd[k].detach().float().cpu()
+    stream, fl = [], []
+    for l in range(n_layers):
+        p = f"encoder.layers.{l}."
+        q_qkv, s_qkv = quantise_weights_int8(get(p + "self_attn.in_proj_weight"))
+        q_out, s_out = quantise_weights_int8(get(p + "self_attn.out_proj.weight"))
+        q_ff1, s_ff1 = quantise_weights_int8(get(p + "linear1.weight"))
+        q_ff2, s_ff2 = quantise_weights_int8(get(p + "linear2.weight"))
+        for h in range(nt):
+            for part in range(3):
+                stream.append(pack_int8_block(q_qkv, part * nt + h, 0))
+        for n in range(nt):
+            stream.append(pack_int8_block(q_out, n, 0))
+        for n in range(ft):
+            stream.append(pack_int8_block(q_ff1, n, 0))
+        for n in range(nt):
+            for c in range(kcf):
+                stream.append(pack_int8_block(q_ff2, n, 256 * c))
+        wsum = (128 * q_ff2.astype(np.int32).reshape(d, kcf, 256).sum(axis=2)).T   # [kcf, d]
+        sw = np.concatenate([s_qkv, s_out, s_ff1, s_ff2]).astype(np.float32)
+        sw = np.concatenate([sw, np.zeros((-len(sw)) % 4, np.float32)])
+        fl += [get(p + "norm1.weight").numpy(), get(p + "norm1.bias").numpy(),
+               get(p + "self_attn.in_proj_bias").numpy(), get(p + "self_attn.out_proj.bias").numpy(),
+               get(p + "norm2.weight").numpy(), get(p + "norm2.bias").numpy(),
+               get(p + "linear1.bias").numpy(), get(p + "linear2.bias").numpy(),
+               np.ascontiguousarray(wsum, dtype=np.int32).view(np.float32).reshape(-1), sw]
+    head = np.zeros((96, d), np.float32)
+    head[:N_POLICY] = get("policy.weight").numpy()
+    head[N_POLICY:N_POLICY + N_PROMO] = get("promo.weight").numpy()
+    head[N_POLICY + N_PROMO:N_POLICY + N_PROMO + n_value] = get("value.weight").numpy()
+    for m in range(3):
+        stream.append(pack_head_tile(head, m).view(np.uint8))
+    for name in ("emb_square", "emb_type_special", "emb_color_turn", "emb_clock", "emb_rep"):
+        fl.append(get(name + ".weight").numpy())
+    fl += [get("norm_f.weight").numpy(), get("norm_f.bias").numpy()]
+    wstream = np.concatenate([s.reshape(-1) for s in stream])
+    fparams = np.concatenate([np.asarray(x, dtype=np.float32).reshape(-1) for x in fl])
+    return wstream, fparams
+
+
+# --------------------------------------------------------------------------- #
+# the evaluator object
+# --------------------------------------------------------------------------- #
+
+class FusedEncoder:
+    """Boards to logits in one launch (see the module docstring)."""
+
+    D, DFF, T, H = 256, 1024, 32, 8
+    ACC_DTYPES = ("fp16", "fp32")
+    n_value = 1
+    vmode = 0
+    rj_mode = 0
+
+    def __init__(self, source, acc_dtype: str = "fp16", fp8: bool = False,
+                 int8: Optional[bool] = None, two_boards: Optional[bool] = None,
+                 int8_scheme: str = "all", out_dtype: torch.dtype = torch.float16,
+                 device: Optional[torch.device] = None):
+        if acc_dtype not in self.ACC_DTYPES:
+            raise ValueError(f"acc_dtype must be one of {self.ACC_DTYPES}, got {acc_dtype!r}")
+        if fp8 and int8:
+            raise ValueError("fp8 and int8 quantise the same matmuls; pick one")
+        if fp8:
+            raise NotImplementedError("this build carries the int8 evaluator only (no e4m3 path yet)")
+        if int8 is False:
+            raise NotImplementedError(
+                "this build carries the int8 evaluator only; construct with int8=True (the default here)")
+        if int8_scheme != "all":
+            raise NotImplementedError(
+                "all four matmuls of every layer are int8 here, which is the reference's 'all' scheme")
+        if out_dtype not in (torch.float16, torch.float32):
+            raise ValueError(f"out_dtype must be float16 or float32, got {out_dtype}")
+        if not hasattr(source, "encoder") or not hasattr(source, "policy"):
+            raise ValueError("forward_full needs the whole model: build this from a BrokefishNet "
+                             "(embeddings, encoder, norm_f and heads), not from a bare encoder stack")
+        if getattr(source, "value_head", "king") != "king" or getattr(source, "reinject", "none") != "none" \
+                or getattr(source, "rule_features", False):
+            raise NotImplementedError("only the king value head without re-injection or rule features")
+        net = source
+        layers = net.encoder.layers
+        first = layers[0]
+        self.n_layers = len(layers)
+        self.d_model = first.self_attn.embed_dim
+        self.n_heads = first.self_attn.num_heads
+        self.d_ff = first.linear1.out_features
+        self.d_head = self.d_model // self.n_heads
+        self.eps = float(first.norm1.eps)
+        if (self.d_model, self.d_ff, self.n_heads) != (self.D, self.DFF, self.H):
+            raise ValueError(
+                f"kernel is compiled for d_model={self.D}, d_ff={self.DFF}, heads={self.H}; "
+                f"got {self.d_model}, {self.d_ff}, {self.n_heads}")
+        if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
+            raise ValueError("the evaluator implements pre-norm ReLU layers only")
+        self.n_value = int(net.value.weight.shape[0])
+        if self.n_value not in (1, 3):
+            raise ValueError(f"value head must have 1 or 3 rows, got {self.n_value}")
+        self.acc_dtype, self.fp8, self.int8 = acc_dtype, False, True
+        self.int8_scheme, self.quant = int8_scheme, 3
+        # Boards per workgroup is an occupancy detail of this kernel (four); the flag is
+        # accepted for signature compatibility and changes no number.
+        self.two_boards = True if two_boards is None else bool(two_boards)
+        self.out_dtype = out_dtype
+        self.net = net
+
+        self._lib = load_library()
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU visible: the evaluator has no CPU path")
+        self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+        self._shape = _Shape(self.d_model, self.n_layers, self.n_heads, self.d_ff, self.n_value, self.eps)
+        sd = {k: v.detach() for k, v in net.state_dict().items()}
+        wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value)
+        if wstream.size != self._lib.bf_wstream_bytes(C.byref(self._shape)) or \
+                fparams.size != self._lib.bf_fparams_floats(C.byref(self._shape)):
+            raise RuntimeError("packed blob sizes disagree with the library's layout")
+        self.wstream = torch.from_numpy(wstream).to(self.device)
+        self.fparams = torch.from_numpy(fparams).to(self.device)
+        self._buffered_full = 0
+        self.best_move = None
+
+    @property
+    def label(self) -> str:
+        return "int8 FFN+QKV+out_proj, 4 boards/workgroup (gfx950)"
+
+    # -- buffers and checks ---------------------------------------------------
+
+    def _ensure_full_buffers(self, n: int) -> None:
+        if self._buffered_full != n:
+            self.policy_out = torch.empty(n, T, N_POLICY, device=self.device, dtype=self.out_dtype)
+            self.promo_out = torch.empty(n, T, N_PROMO, device=self.device, dtype=self.out_dtype)
+            self.value_out = torch.empty(n, device=self.device, dtype=torch.float32)
+            self.best_out = torch.empty(n, device=self.device, dtype=torch.int32)
+            self._buffered_full = n
+
+    @staticmethod
+    def _check_inputs(boards, control, rep, mask=None) -> int:
+        if boards.dim() != 2 or boards.shape[1] != T:
+            raise ValueError(f"boards must be [n, 32], got {tuple(boards.shape)}")
+        n = boards.shape[0]
+        if n < 1:
+            raise ValueError("boards must hold at least one position")
+        if boards.dtype is not torch.int16:
+            raise ValueError(f"boards must be int16, got {boards.dtype}")
+        if control.shape != (n,) or control.dtype is not torch.int16:
+            raise ValueError(f"control must be [{n}] int16, got {tuple(control.shape)} {control.dtype}")
+        if rep.shape != (n,) or rep.dtype is not torch.uint8:
+            raise ValueError(f"rep must be [{n}] uint8, got {tuple(rep.shape)} {rep.dtype}")
+        if mask is not None and (mask.shape != (n, T) or mask.dtype is not torch.int64):
+            raise ValueError(f"mask must be [{n}, 32] int64, got {tuple(mask.shape)} {mask.dtype}")
+        for name, t in (("boards", boards), ("control", control), ("rep", rep), ("mask", mask)):
+            if t is not None and not t.is_cuda:
+                raise ValueError(f"{name} must be on the GPU")
+        return n
+
+    def _args(self, boards, control, rep, mask, policy, promo, value, best, taps=None) -> _Args:
+        a = _Args()
+        a.boards, a.control, a.rep = boards.data_ptr(), control.data_ptr(), rep.data_ptr()
+        a.mask = mask.data_ptr() if mask is not None else None
+        a.n = boards.shape[0]
+        a.shape = self._shape
+        a.wstream, a.fparams = self.wstream.data_ptr(), self.fparams.data_ptr()
+        a.policy, a.promo, a.value = policy.data_ptr(), promo.data_ptr(), value.data_ptr()
+        a.best_move = best.data_ptr() if (best is not None and mask is not None) else None
+        a.out_fp32 = 1 if policy.dtype is torch.float32 else 0
+        a.taps = C.pointer(taps) if taps is not None else None
+        return a
+
+    def _call(self, args: _Args) -> None:
+        rc = self._lib.bf_model_forward(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream))
+        if rc:
+            raise RuntimeError(f"bf_model_forward failed ({rc}): {self._lib.bf_last_error().decode()}")
+
+    # -- the call ----------------------------------------------------------------
+
+    def forward_full(self, boards, control, rep, mask=None):
+        """Boards to ``(policy_logits, promo, value)`` in one launch.
+
+        Without ``mask`` the policy is raw, as the reference evaluator returns it.  With
+        ``mask`` illegal entries are ``-inf`` and ``self.best_move`` ([n] int32) is the
+        masked argmax.  Returns views on internal buffers, which the next call overwrites.
+        """
+        n = self._check_inputs(boards, control, rep, mask)
+        self._ensure_full_buffers(n)
+        boards, control, rep = boards.contiguous(), control.contiguous(), rep.contiguous()
+        mask = mask.contiguous() if mask is not None else None
+        self._call(self._args(boards, control, rep, mask, self.policy_out, self.promo_out,
+                              self.value_out, self.best_out))
+        self.best_move = self.best_out if mask is not None else None
+        return self.policy_out, self.promo_out, self.value_out
+
+    def forward_masked(self, boards, control, rep, mask):
+        """``(policy_logits, promo, value, best_move)`` with the legal-move AND fused in."""
+        p, q, v = self.forward_full(boards, control, rep, mask)
+        return p, q, v, self.best_out
+
+    def time_kernel_ms(self, boards, control, rep, mask=None, warmup: int = 3, iters: int = 20) -> float:
+        """Average device time of one launch, from HIP events on the current stream."""
+        n = self._check_inputs(boards, control, rep, mask)
+        self._ensure_full_buffers(n)
+        args = self._args(boards.contiguous(), control.contiguous(), rep.contiguous(),
+                          mask.contiguous() if mask is not None else None,
+                          self.policy_out, self.promo_out, self.value_out, self.best_out)
+        ms = self._lib.bf_time_kernel_ms(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
+                                         warmup, iters)
+        if ms < 0:
+            raise RuntimeError(f"bf_time_kernel_ms failed ({ms}): {self._lib.bf_last_error().decode()}")
+        return ms
+
+    # -- debug taps (the counterpart of the reference's forward_stage) ------------
+
+    def forward_taps(self, boards, control, rep, mask=None, x_in=None, layer_begin: int = 0,
+                     layer_end: Optional[int] = None, want=None):
+        """Run with intermediate outputs.  Returns a dict of fresh fp32-output tensors:
+        policy, promo, value, [best], plus the taps named in ``want`` (default: all).
+
+        ``x_in`` ([n,32,d] fp32) replaces the embedding as the residual stream entering
+        layer ``layer_begin``; layers ``[layer_begin, layer_end)`` run, then the heads.
+        """
+        n = self._check_inputs(boards, control, rep, mask)
+        d, f = self.d_model, self.d_ff
+        layer_end = self.n_layers if layer_end is None else layer_end
+        lr = layer_end - layer_begin
+        kd, kf = d // 256, f // 256
+        dev = self.device
+        shapes = {"embed": ((n, T, d), torch.float32),
+                  "qa_qkv": ((n, lr, T, d), torch.int8), "acc_qkv": ((n, lr, kd, T, 3 * d), torch.int32),
+                  "qa_out": ((n, lr, T, d), torch.int8), "acc_out": ((n, lr, kd, T, d), torch.int32),
+                  "qa_ff1": ((n, lr, T, d), torch.int8), "acc_ff1": ((n, lr, kd, T, f), torch.int32),
+                  "qa_ff2": ((n, lr, T, f), torch.uint8), "acc_ff2": ((n, lr, kf, T, d), torch.int32),
+                  "resid": ((n, lr, T, d), torch.float32), "normed": ((n, T, d), torch.float32)}
+        want = list(shapes) if want is None else list(want)
+        out = {k: torch.zeros(shapes[k][0], dtype=shapes[k][1], device=dev) for k in want}
+        taps = _Taps()
+        if x_in is not None:
+            if x_in.shape != (n, T, d) or x_in.dtype is not torch.float32 or not x_in.is_cuda:
+                raise ValueError(f"x_in must be [{n}, 32, {d}] float32 on the GPU")
+            x_in = x_in.contiguous()
+            taps.x_in = x_in.data_ptr()
+        taps.layer_begin, taps.layer_end = layer_begin, layer_end
+        if layer_begin == 0 and layer_end == 0:
+            raise ValueError("empty layer range")
+        for k in want:
+            setattr(taps, k, out[k].data_ptr())
+        out["policy"] = torch.empty(n, T, N_POLICY, device=dev, dtype=torch.float32)
+        out["promo"] = torch.empty(n, T, N_PROMO, device=dev, dtype=torch.float32)
+        out["value"] = torch.empty(n, device=dev, dtype=torch.float32)
+        best = torch.empty(n, device=dev, dtype=torch.int32) if mask is not None else None
+        if best is not None:
+            out["best"] = best
+        self._call(self._args(boards.contiguous(), control.contiguous(), rep.contiguous(),
+                              mask.contiguous() if mask is not None else None,
+                              out["policy"], out["promo"], out["value"], best, taps))
+        torch.cuda.current_stream(dev).synchronize()   # taps/x_in must outlive the launch
+        return out

@@ -1,0 +1,146 @@
+/* C-ABI of the MI355X (gfx950) network evaluator: packed board words in, policy /
+ * promotion logits and value out, one kernel launch.
+ *
+ * This is the boundary a host binds in place of the reference's CUDA extension module
+ * (reference csrc/encoder.cu:1905-1930 lists the functions that module exports).  Plain
+ * pointers and sizes only; every pointer is a DEVICE pointer unless stated otherwise.
+ * Nothing here allocates, frees or synchronises: outputs are caller-allocated and the
+ * launch is asynchronous on the stream that is passed in.
+ *
+ * Functions return 0 on success, a negative bf_status on rejected arguments (nothing is
+ * launched then) and bf_last_error() describes the most recent failure of the calling
+ * thread.
+ */
+#ifndef BROKEFISH_HIP_H
+#define BROKEFISH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum bf_status {
+    BF_OK = 0,
+    BF_ERR_ARGUMENT = -1,   /* null / misaligned pointer, bad size or mode */
+    BF_ERR_UNSUPPORTED = -2, /* network shape this build has no kernel for */
+    BF_ERR_LAUNCH = -3,     /* hipLaunchKernel reported an error */
+    BF_ERR_DEVICE = -4      /* not a gfx950 device */
+};
+
+/* Sizes of one 32-token position, fixed by the position format
+ * (reference docs/reference/spec.md:94-106). */
+#define BF_TOKENS 32
+#define BF_POLICY 64
+#define BF_PROMO 4
+
+/* Network shape.  Supported: d_model 256, n_heads 8 (head width 32), d_ff 1024, any
+ * n_layers >= 1, n_value 1 (tanh scalar) or 3 (loss/draw/win classes). */
+typedef struct {
+    int32_t d_model, n_layers, n_heads, d_ff, n_value;
+    float eps;
+} bf_shape;
+
+/* Layout queries for the two parameter blobs the host packs (see the layout section at
+ * the end of this header).  Return 0 for an unsupported shape. */
+size_t bf_wstream_bytes(const bf_shape* s);   /* int8 weight tiles + fp32 head tiles */
+size_t bf_fparams_floats(const bf_shape* s);  /* fp32 / int32 side parameters        */
+
+/* Optional debug outputs ("taps") and teacher forcing.  All pointers may be NULL.
+ * B = boards in the call, L = layers run, kc = K / 256.
+ * Replaces the reference's debug_stage / forward_stage mechanism
+ * (reference brokefish/nn/cuda_impl.py:512-531, csrc/encoder.cu:1575-1598). */
+typedef struct {
+    const float* x_in;  /* [B,32,d] residual stream to start from instead of the embedding */
+    int32_t layer_begin, layer_end; /* run layers [begin, end); 0,0 means all */
+    float* embed;       /* [B,32,d]  embedding sum (or x_in echoed)                */
+    int8_t* qa_qkv;     /* [B,L,32,d]    operand bytes fed to the QKV matmul       */
+    int32_t* acc_qkv;   /* [B,L,kc,32,3d] its int32 accumulators                   */
+    int8_t* qa_out;     /* [B,L,32,d]                                              */
+    int32_t* acc_out;   /* [B,L,kc,32,d]                                           */
+    int8_t* qa_ff1;     /* [B,L,32,d]                                              */
+    int32_t* acc_ff1;   /* [B,L,kc,32,d_ff]                                        */
+    uint8_t* qa_ff2;    /* [B,L,32,d_ff] unsigned operand bytes of the second FFN matmul */
+    int32_t* acc_ff2;   /* [B,L,kc,32,d] accumulators of the unsigned product      */
+    float* resid;       /* [B,L,32,d] residual stream after each layer             */
+    float* normed;      /* [B,32,d]   after the final LayerNorm                    */
+} bf_taps;
+
+typedef struct {
+    /* inputs (reference csrc/encoder.cu:1770-1790: boards [n,32] int16, control [n]
+     * int16, rep [n] uint8, contiguous, on the device) */
+    const uint16_t* boards;
+    const int16_t* control;
+    const uint8_t* rep;
+    /* optional legal-move words [n,32], bit s of word p set iff p -> s is legal
+     * (reference docs/reference/spec.md:141-143).  NULL = raw logits, as the
+     * reference evaluator returns them (docs/reference/spec.md:527-535). */
+    const uint64_t* mask;
+    int64_t n;
+    /* parameters */
+    bf_shape shape;
+    const uint8_t* wstream;
+    const float* fparams;
+    /* outputs: policy [n,32,64], promo [n,32,4] in fp16 (out_fp32 = 0, the search
+     * contract of reference brokefish/nn/cuda_impl.py:467-472) or fp32; value [n] fp32
+     * in [-1,1].  With a mask, illegal policy entries are -inf and best_move [n]
+     * (optional) receives slot*64+square of the largest legal logit, lowest index on
+     * ties, -1 when no move is legal. */
+    void* policy;
+    void* promo;
+    float* value;
+    int32_t* best_move;
+    int32_t out_fp32;
+    const bf_taps* taps; /* NULL in production */
+} bf_eval_args;
+
+/* The evaluator.  Replaces model_forward of the reference extension
+ * (reference csrc/encoder.cu:1770-1876, bound at :1918-1925; called from
+ * brokefish/nn/cuda_impl.py:497-503).  `stream` is a hipStream_t (NULL = default). */
+int bf_model_forward(const bf_eval_args* args, void* stream);
+
+/* Quantisation maxima of the signed / unsigned activation formats, for the host to pin
+ * against its own constants.  Replaces int8_q_max (reference csrc/encoder.cu:1926-1929). */
+void bf_int8_q_max(double* s8, double* u8);
+
+/* Message for the last non-zero status returned to this thread. */
+const char* bf_last_error(void);
+
+/* Average device time of the evaluator kernel, measured with HIP events recorded on
+ * `stream` around `iters` back-to-back launches (after `warmup` launches).  Returns
+ * milliseconds per launch, or a negative bf_status.  Synchronises the stream.
+ * Stands in for the reference's in-kernel phase profile hooks
+ * (reference csrc/encoder.cu:1886-1903) at whole-kernel granularity. */
+double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int iters);
+
+/* -------------------------------------------------------------------------------------
+ * Blob layouts (what the host packer writes; brokefish_amd/hip_impl.py is the packer).
+ *
+ * Lane order: within a 32-wide tile, lane half g (0/1) and index r (0..15) address
+ *     ch(r, g) = 8 * (r / 4) + 4 * g + (r % 4).
+ *
+ * wstream: a sequence of 1 KiB fragments; a fragment holds 64 lanes x 16 bytes.  For an
+ * int8 fragment of output tile n and k-step s of matrix W [N, K] (rows = output
+ * channels), lane = 32 * g + o holds W[32 n + o][k0 + 32 s + ch(r, g)] at byte r.
+ * 8 fragments (s = 0..7, one 256-wide k-chunk) make a block; per layer the blocks are
+ *     for head h:  Q tile h, K tile h, V tile h        (rows h*32, d + h*32, 2d + h*32)
+ *     out-proj tiles 0..7
+ *     ffn1 tiles 0..31
+ *     for ffn2 output tile n: for k-chunk c = 0..3: block (n, c)
+ * and after the last layer three 32 KiB fp32 head tiles: head tile m (rows 32m..32m+31
+ * of [policy(64); promo(4); value(n_value); zeros]), fragment (n, q), lane 32g + o holds
+ * the four floats W[32 m + o][32 n + 8 q + 4 g + 0..3].
+ *
+ * fparams (fp32 unless noted), per layer at stride bf_layer_floats:
+ *     ln1_gamma[d] ln1_beta[d] b_qkv[3d] b_out[d] ln2_gamma[d] ln2_beta[d] b_ffn1[f]
+ *     b_ffn2[d] wsum[kc_f][d] (int32: 128 * sum of the int8 weights of ffn2 row over
+ *     k-chunk c) sw_qkv[3d/128] sw_out[d/128] sw_ffn1[f/128] sw_ffn2[d/128]
+ * then the five embedding tables (square 64, type_special 12, color_turn 4, clock 101,
+ * rep 3 rows of d) and norm_f gamma[d], beta[d].
+ * ----------------------------------------------------------------------------------- */
+
+#ifdef __cplusplus
+}
+#endif
+#endif

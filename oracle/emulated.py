@@ -1,0 +1,186 @@
+"""TEST INFRASTRUCTURE -- NOT PRODUCT CODE.
+
+A CPU restatement, in plain PyTorch library calls, of the reference network forward in
+its two modes: fp32, and the int8-simulated forward the HIP evaluator must reproduce.
+Only ``tests/``, ``__graft_entry__.smoke()`` and ``bench.py``'s CPU-baseline leg import
+this module; nothing under ``brokefish_amd/`` does.
+
+It works on a bare ``state_dict`` (same key names as the reference model,
+brokefish/nn/model.py:297-316), so it does not depend on any model class.
+
+What each function follows (paths inside the reference tree):
+
+* :func:`decode_words`, :func:`embed_indices`  -- brokefish/nn/model.py:251-265, :455-477
+* :func:`embed`                                 -- brokefish/nn/model.py:635-640 (order normative,
+  docs/reference/spec.md:386-391)
+* :func:`quantise_activations_int8`             -- brokefish/nn/quant.py:246-260
+* :func:`quantise_weights_int8`                 -- brokefish/nn/quant.py:263-278
+* :func:`int8_linear`                           -- brokefish/nn/quant.py:281-305
+* :func:`forward` block structure               -- torch ``TransformerEncoderLayer(norm_first=True)``
+  as constructed at brokefish/nn/model.py:303-311 and called at :525 with
+  ``src_key_padding_mask=~alive``; the four matmuls routed through ``int8_linear`` and
+  ``ffn2`` unsigned as in brokefish/nn/quant.py:421-440, :466-473
+* heads                                         -- brokefish/nn/model.py:551-617
+* mask AND / argmax (not in the reference evaluator; the search applies it)
+                                                -- docs/reference/spec.md:141-143, :537-540
+
+LayerNorm, softmax and the fp32 matmuls are torch library routines here, so their
+summation order is torch's; the C checker ``bf_oracle.c`` fixes explicit orders instead.
+The two agree to rounding noise, which ``tests/test_oracle.py`` asserts.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+import torch.nn.functional as F
+
+ROW_K = 256      # brokefish/nn/quant.py:92
+BLOCK_N = 128    # brokefish/nn/quant.py:82
+Q_MAX_S8 = 127.0  # brokefish/nn/quant.py:237
+Q_MAX_U8 = 255.0  # brokefish/nn/quant.py:241
+KING_WHITE, KING_BLACK = 15, 31
+
+
+def decode_words(boards: torch.Tensor):
+    w = boards.to(torch.int64) & 0xFFFF
+    return (w >> 11) & 1, (w >> 10) & 1, (w >> 9) & 1, (w >> 6) & 7, w & 63
+
+
+def embed_indices(boards, control, rep):
+    captured, colour, special, ptype, square = decode_words(boards)
+    stm = (control < 0).to(torch.int64)
+    clock = (control.to(torch.int64).abs() - 1).clamp(0, 100)
+    return (square, ptype * 2 + special, colour * 2 + stm[:, None], clock,
+            rep.to(torch.int64).clamp(0, 2)), captured == 0
+
+
+def embed(sd: Dict[str, torch.Tensor], boards, control, rep):
+    idx, alive = embed_indices(boards, control, rep)
+    per_board = sd["emb_clock.weight"][idx[3]] + sd["emb_rep.weight"][idx[4]]
+    x = sd["emb_square.weight"][idx[0]]
+    x = x + sd["emb_type_special.weight"][idx[1]]
+    x = x + sd["emb_color_turn.weight"][idx[2]]
+    x = x + per_board[:, None, :]
+    return x, alive
+
+
+def quantise_activations_int8(x: torch.Tensor, unsigned: bool = False):
+    """[M, K] fp32 -> (integer-valued fp32 [M, K], scale [M, 1])."""
+    if unsigned:
+        pos = x.clamp(min=0)
+        amax = pos.amax(dim=-1, keepdim=True)
+        s = torch.where(amax > 0, amax / Q_MAX_U8, torch.ones_like(amax))
+        return torch.round(pos / s).clamp(0, Q_MAX_U8), s
+    amax = x.abs().amax(dim=-1, keepdim=True)
+    s = torch.where(amax > 0, amax / Q_MAX_S8, torch.ones_like(amax))
+    return torch.round(x / s).clamp(-Q_MAX_S8, Q_MAX_S8), s
+
+
+def quantise_weights_int8(w: torch.Tensor):
+    """[N, K] fp32 -> (int8 [N, K], scale [N // 128]); one scale per 128 output rows."""
+    n, k = w.shape
+    if n % BLOCK_N:
+        raise ValueError(f"weight {tuple(w.shape)} does not tile into {BLOCK_N} rows")
+    blocks = w.float().reshape(n // BLOCK_N, BLOCK_N * k)
+    amax = blocks.abs().amax(dim=1, keepdim=True)
+    s = torch.where(amax > 0, amax / Q_MAX_S8, torch.ones_like(amax))
+    q = torch.round(blocks / s).clamp(-Q_MAX_S8, Q_MAX_S8).to(torch.int8)
+    return q.reshape(n, k), s.reshape(-1).contiguous()
+
+
+def int8_linear(x, w, bias, unsigned: bool = False, taps: Optional[dict] = None, name: str = ""):
+    """``F.linear`` with both operands int8, exact integer accumulation per 256-wide
+    k-chunk, float64 across chunks, one weight descale at the end."""
+    lead = x.shape[:-1]
+    a = x.reshape(-1, x.shape[-1]).float()
+    m, k = a.shape
+    n = w.shape[0]
+    wq, ws = quantise_weights_int8(w)
+    wq64 = wq.to(torch.float64)
+    out = torch.zeros(m, n, dtype=torch.float64)
+    qs, accs = [], []
+    for lo in range(0, k, ROW_K):
+        q, sa = quantise_activations_int8(a[:, lo:lo + ROW_K], unsigned)
+        acc = q.to(torch.float64) @ wq64[:, lo:lo + ROW_K].T
+        out += acc * sa.to(torch.float64)
+        if taps is not None:
+            qs.append(q.to(torch.int16))
+            accs.append(acc.to(torch.int32))
+    if taps is not None:
+        taps.setdefault("qa_" + name, []).append(torch.cat(qs, dim=1))
+        taps.setdefault("acc_" + name, []).append(torch.stack(accs))
+    y = out.to(torch.float32) * ws.repeat_interleave(BLOCK_N)[None, :]
+    if bias is not None:
+        y = y + bias.float()
+    return y.reshape(*lead, n)
+
+
+def _linear(x, w, b, mode, unsigned=False, taps=None, name=""):
+    if mode == "int8":
+        return int8_linear(x, w, b, unsigned, taps, name)
+    return F.linear(x, w, b)
+
+
+def n_layers_of(sd) -> int:
+    n = 0
+    while f"encoder.layers.{n}.linear1.weight" in sd:
+        n += 1
+    return n
+
+
+def forward(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8",
+            mask: Optional[torch.Tensor] = None, n_heads: Optional[int] = None,
+            eps: float = 1e-5, taps: Optional[dict] = None):
+    """(policy [N,32,64], promo [N,32,4], value [N]) in fp32, plus ``best`` [N] int64
+    (slot*64+square of the masked argmax) when ``mask`` is given.
+
+    ``mode`` is ``"fp32"`` (every matmul an ordinary ``F.linear``) or ``"int8"`` (the
+    four body matmuls of every layer through :func:`int8_linear`).
+    """
+    if mode not in ("fp32", "int8"):
+        raise ValueError(mode)
+    x, alive = embed(sd, boards, control, rep)
+    n, t, d = x.shape
+    heads = n_heads if n_heads is not None else d // 32
+    dh = d // heads
+    if taps is not None:
+        taps["embed"] = x.clone()
+    key_bias = torch.zeros(n, 1, 1, t)
+    key_bias.masked_fill_(~alive[:, None, None, :], float("-inf"))
+    for i in range(n_layers_of(sd)):
+        p = f"encoder.layers.{i}."
+        y = F.layer_norm(x, (d,), sd[p + "norm1.weight"], sd[p + "norm1.bias"], eps)
+        qkv = _linear(y, sd[p + "self_attn.in_proj_weight"], sd[p + "self_attn.in_proj_bias"],
+                      mode, False, taps, "qkv")
+        q, k, v = (z.reshape(n, t, heads, dh).transpose(1, 2) for z in qkv.split(d, dim=-1))
+        s = (q @ k.transpose(-1, -2)) * (1.0 / math.sqrt(dh)) + key_bias
+        o = (torch.softmax(s, dim=-1) @ v).transpose(1, 2).reshape(n, t, d)
+        x = x + _linear(o, sd[p + "self_attn.out_proj.weight"], sd[p + "self_attn.out_proj.bias"],
+                        mode, False, taps, "out")
+        y = F.layer_norm(x, (d,), sd[p + "norm2.weight"], sd[p + "norm2.bias"], eps)
+        hid = torch.relu(_linear(y, sd[p + "linear1.weight"], sd[p + "linear1.bias"],
+                                 mode, False, taps, "ff1"))
+        x = x + _linear(hid, sd[p + "linear2.weight"], sd[p + "linear2.bias"],
+                        mode, True, taps, "ff2")
+        if taps is not None:
+            taps.setdefault("resid", []).append(x.clone())
+    h = F.layer_norm(x, (d,), sd["norm_f.weight"], sd["norm_f.bias"], eps)
+    if taps is not None:
+        taps["normed"] = h.clone()
+    policy = F.linear(h, sd["policy.weight"])
+    promo = F.linear(h, sd["promo.weight"])
+    king = torch.where(control < 0, KING_BLACK, KING_WHITE).to(torch.int64)
+    raw = F.linear(h[torch.arange(n), king], sd["value.weight"]).float()
+    if raw.shape[-1] == 1:
+        value = torch.tanh(raw).squeeze(-1)
+    else:  # classes 0 = loss, 1 = draw, 2 = win from the side to move
+        pr = torch.softmax(raw, dim=-1)
+        value = pr[:, 2] - pr[:, 0]
+    if mask is None:
+        return policy, promo, value
+    legal = ((mask.to(torch.int64)[..., None] >> torch.arange(64)) & 1).bool()
+    policy = policy.masked_fill(~legal, float("-inf"))
+    best = policy.reshape(n, -1).argmax(dim=1)   # torch.argmax returns the first maximum
+    return policy, promo, value, best
