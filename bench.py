@@ -1,0 +1,111 @@
+"""Headline benchmark: network evaluations per second at batch 4096, int8, one MI355X.
+
+One step = one launch of the evaluator over one batch of synthetic positions (seeded
+random playouts of 0-120 plies, with legal-move masks ANDed in-kernel); inputs are resident
+in HBM and outputs preallocated before the timed region.  Prints ONE JSON line.
+
+Extra objects in the line:
+  roofline      dense-int8 MFMA roofline of the evaluator kernel: algorithmic int8 ops per
+                launch (402,653,184 per evaluation x batch) over the kernel's average duration
+                measured with HIP events on the launch stream.
+  cpu_baseline  the CPU port of the same forward (oracle/emulated.py, PyTorch on the host
+                cores) timed on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+OPS_PER_EVAL = 402_653_184            # 2 * 32 tokens * 8 layers * 12 * 256^2 int8 ops in the weight GEMMs
+PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s
+
+
+def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0):
+    """The int8-simulated forward of oracle/emulated.py on the host cores (a port, not the
+    reference's files, which do not travel)."""
+    import torch
+    from brokefish_amd import positions
+    from oracle import emulated
+    sd = {k: v.detach() for k, v in net.state_dict().items()}
+    b, c, r, m = positions.random_positions(batch, plies=120, seed=0)
+    torch.set_num_threads(threads)
+    with torch.no_grad():
+        t0 = time.perf_counter()
+        emulated.forward(sd, b, c, r, mode="int8", mask=m)             # warm-up, also sizes the loop
+        one = time.perf_counter() - t0
+        reps = max(2, min(20, int(budget_s / max(one, 1e-3))))
+        times = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            emulated.forward(sd, b, c, r, mode="int8", mask=m)
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": batch / med, "unit": "evals/s", "cores": threads, "kind": "port",
+            "sample": f"{reps} reps of batch {batch} (int8-simulated PyTorch forward, median), "
+                      f"os.cpu_count()={os.cpu_count()}"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=4096)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-batch", type=int, default=64)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this path runs on one GPU (positions shard with no exchange step); --gpus must be 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    from brokefish_amd import encoder_impl, positions
+    from brokefish_amd.net import BrokefishNet
+
+    torch.manual_seed(0)
+    net = BrokefishNet().eval()                                  # seed-0 random init, reference init rules
+    model = encoder_impl("hip")(net, int8=True)                  # fp16 logits: the search contract
+    b, c, r, m = positions.random_positions(a.batch, plies=120, seed=0)
+    bd, cd, rd, md = b.cuda(), c.cuda(), r.cuda(), m.cuda()
+
+    for _ in range(a.warmup):
+        model.forward_full(bd, cd, rd, md)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        model.forward_full(bd, cd, rd, md)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_step = dt / a.steps * 1e3
+    evals = a.batch * a.steps / dt
+
+    kern_ms = model.time_kernel_ms(bd, cd, rd, md, warmup=3, iters=max(a.steps, 10))
+    achieved = OPS_PER_EVAL * a.batch / (kern_ms * 1e-3) / 1e12
+    line = {
+        "metric": "network evals/sec at batch 4096 int8 on 1 MI355X",
+        "value": evals, "unit": "evals/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": f"configs[1]: 8-layer d256 8-head FFN1024 int8 evaluator, batch {a.batch}, "
+                               "seeded random playouts 0-120 plies, legal-move mask ANDed in-kernel, "
+                               "fp16 logits out, seed-0 random-init weights"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
+                     "frac": achieved / (PEAK_INT8_OPS / 1e12), "traffic": None,
+                     "kernel_ms": kern_ms, "ops_per_launch": OPS_PER_EVAL * a.batch},
+    }
+    if not a.no_cpu:
+        threads = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+        line["cpu_baseline"] = cpu_baseline(net, a.cpu_batch, threads)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

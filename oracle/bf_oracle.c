@@ -373,6 +373,9 @@ int bfo_forward(const bfo_model* m, const uint16_t* boards, const int16_t* contr
     const int nv = m->cfg.n_value;
     const float eps = m->cfg.eps;
     const int kc_d = d / ROW_K, kc_f = f / ROW_K;
+    int l0 = 0, l1 = L;
+    if (taps && (taps->layer_begin || taps->layer_end)) { l0 = taps->layer_begin; l1 = taps->layer_end; }
+    if (l0 < 0 || l1 > L || l0 > l1) return -1;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int b = 0; b < n; b++) {
         float* x = (float*)malloc((size_t)T * d * 4);
@@ -386,9 +389,10 @@ int bfo_forward(const bfo_model* m, const uint16_t* boards, const int16_t* contr
         int32_t* acc = (int32_t*)malloc((size_t)T * (size_t)(3 * d > f ? 3 * d : f) * (kc_f > kc_d ? kc_f : kc_d) * 4);
 
         const uint32_t alive = embed_board(m, boards + (size_t)b * 32, control[b], rep[b], x);
+        if (taps && taps->x_in) memcpy(x, taps->x_in + (size_t)b * T * d, (size_t)T * d * 4);
         if (taps && taps->embed) memcpy(taps->embed + (size_t)b * T * d, x, (size_t)T * d * 4);
-        for (int l = 0; l < L; l++) {
-            const size_t bl = (size_t)b * L + l;
+        for (int l = l0; l < l1; l++) {
+            const size_t bl = (size_t)b * (l1 - l0) + (l - l0);
             /* x += out_proj(attention(in_proj(LN1(x)))) */
             layernorm_rows(x, d, m->norm1_w + (size_t)l * d, m->norm1_b + (size_t)l * d, eps, y);
             bfo_int8_linear_q(y, T, d, m->q_qkv + (size_t)l * 3 * d * d, m->s_qkv + (size_t)l * (3 * d / 128),

@@ -30,6 +30,8 @@ typedef struct {
  *   qa_*   int8 operand bytes exactly as quantised (u8 bit patterns for ffn2)
  *   acc_*  exact integer accumulators, [B, L, kc, 32, Nout] */
 typedef struct {
+    const float* x_in; /* [B,32,d] residual stream to start from instead of the embedding */
+    int layer_begin, layer_end; /* run layers [begin, end); 0,0 means all.  L below = layers run */
     float* embed;      /* [B,32,d] */
     int8_t* qa_qkv;    /* [B,L,32,d] */
     int32_t* acc_qkv;  /* [B,L,kc,32,3d] */

@@ -46,7 +46,8 @@ _TAP_FIELDS = ["embed", "qa_qkv", "acc_qkv", "qa_out", "acc_out", "qa_ff1", "acc
 
 
 class _Taps(C.Structure):
-    _fields_ = [(n, C.c_void_p) for n in _TAP_FIELDS]
+    _fields_ = ([("x_in", C.c_void_p), ("layer_begin", C.c_int), ("layer_end", C.c_int)]
+                + [(n, C.c_void_p) for n in _TAP_FIELDS])
 
 
 _lib = None
@@ -176,8 +177,8 @@ class COracle:
             raise ValueError("unsupported dimensions for the C checker")
 
     def __del__(self):
-        if getattr(self, "_h", None):
-            lib().bfo_model_destroy(self._h)
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.bfo_model_destroy(self._h)
             self._h = None
 
     def qweight(self, which: str, layer: int):
@@ -191,13 +192,19 @@ class COracle:
         s = np.ctypeslib.as_array(C.cast(sp, C.POINTER(C.c_float)), shape=(n // 128,)).copy()
         return q, s
 
-    def forward(self, boards, control, rep, mask=None, taps: bool = False):
-        """numpy in, dict of numpy out: policy, promo, value, [best], [taps...]."""
+    def forward(self, boards, control, rep, mask=None, taps: bool = False, x_in=None,
+                layer_begin: int = 0, layer_end: Optional[int] = None):
+        """numpy in, dict of numpy out: policy, promo, value, [best], [taps...].
+
+        ``x_in`` ([n,32,d] fp32) replaces the embedding as the residual stream entering
+        ``layer_begin``; layers ``[layer_begin, layer_end)`` run, then the heads."""
         b = np.ascontiguousarray(np.asarray(boards).astype(np.int16).view(np.uint16))
         c = np.ascontiguousarray(np.asarray(control), dtype=np.int16)
         r = np.ascontiguousarray(np.asarray(rep), dtype=np.uint8)
         n = b.shape[0]
-        d, L, f = self.d, self.L, self.f
+        d, f = self.d, self.f
+        layer_end = self.L if layer_end is None else layer_end
+        L = layer_end - layer_begin
         out = {"policy": np.empty((n, 32, 64), np.float32), "promo": np.empty((n, 32, 4), np.float32),
                "value": np.empty(n, np.float32)}
         mk = None
@@ -207,7 +214,11 @@ class COracle:
             best = np.empty(n, np.int32)
             out["best"] = best
         tp = None
-        if taps:
+        xin = None
+        if x_in is not None:
+            xin = _f32(x_in)
+            assert xin.shape == (n, 32, d)
+        if taps or xin is not None:
             kd, kf = d // 256, f // 256
             t = {"embed": np.empty((n, 32, d), np.float32),
                  "qa_qkv": np.empty((n, L, 32, d), np.int8), "acc_qkv": np.empty((n, L, kd, 32, 3 * d), np.int32),
@@ -215,8 +226,11 @@ class COracle:
                  "qa_ff1": np.empty((n, L, 32, d), np.int8), "acc_ff1": np.empty((n, L, kd, 32, f), np.int32),
                  "qa_ff2": np.empty((n, L, 32, f), np.int8), "acc_ff2": np.empty((n, L, kf, 32, d), np.int32),
                  "resid": np.empty((n, L, 32, d), np.float32), "normed": np.empty((n, 32, d), np.float32)}
-            out.update(t)
-            tp = _Taps(**{k: v.ctypes.data for k, v in t.items()})
+            if taps:
+                out.update(t)
+            tp = _Taps(**({k: v.ctypes.data for k, v in t.items()} if taps else {}))
+            tp.x_in = xin.ctypes.data if xin is not None else None
+            tp.layer_begin, tp.layer_end = layer_begin, layer_end
         rc = lib().bfo_forward(self._h, b.ctypes.data, c.ctypes.data, r.ctypes.data,
                                mk.ctypes.data if mk is not None else None, n,
                                out["policy"].ctypes.data, out["promo"].ctypes.data, out["value"].ctypes.data,

@@ -184,3 +184,70 @@ def forward(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8
     policy = policy.masked_fill(~legal, float("-inf"))
     best = policy.reshape(n, -1).argmax(dim=1)   # torch.argmax returns the first maximum
     return policy, promo, value, best
+
+
+def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8",
+                          n_heads: Optional[int] = None, eps: float = 1e-5):
+    """The same forward, but with the encoder stack run by torch's own
+    ``nn.TransformerEncoder`` / ``nn.MultiheadAttention`` modules, exactly the modules the
+    reference model is built from (brokefish/nn/model.py:303-311).
+
+    In ``"int8"`` mode the four body matmuls of every layer are diverted to
+    :func:`int8_linear` by intercepting ``torch.nn.functional.linear`` for precisely those
+    weight tensors (the only hook torch's attention module offers for its packed QKV and
+    output projections), with the attention fast path switched off so the module really
+    calls ``F.linear``; ``linear2`` gets the unsigned quantiser.  Under the torch version
+    that wrote ``tests/golden/reference_vectors.npz`` this reproduces the reference's
+    emulated forward bit for bit, which is what pins the composition.
+    """
+    from torch import nn
+
+    x, alive = embed(sd, boards, control, rep)
+    d = x.shape[-1]
+    heads = n_heads if n_heads is not None else d // 32
+    n_layers = n_layers_of(sd)
+    f = sd["encoder.layers.0.linear1.weight"].shape[0]
+    layer = nn.TransformerEncoderLayer(d_model=d, nhead=heads, dim_feedforward=f, batch_first=True,
+                                       norm_first=True, dropout=0.0, layer_norm_eps=eps)
+    stack = nn.TransformerEncoder(layer, num_layers=n_layers, norm=None, enable_nested_tensor=False).eval()
+    stack.load_state_dict({k[len("encoder."):]: v for k, v in sd.items() if k.startswith("encoder.")})
+    unsigned_of = {}
+    for lay in stack.layers:
+        unsigned_of[id(lay.self_attn.in_proj_weight)] = False
+        unsigned_of[id(lay.self_attn.out_proj.weight)] = False
+        unsigned_of[id(lay.linear1.weight)] = False
+        unsigned_of[id(lay.linear2.weight)] = True
+    plain_linear = F.linear
+    hits = [0]
+
+    def routed(inp, weight, bias=None):
+        u = unsigned_of.get(id(weight))
+        if u is None or mode != "int8":
+            return plain_linear(inp, weight, bias)
+        hits[0] += 1
+        return int8_linear(inp, weight, bias, unsigned=u)
+
+    fast = torch.backends.mha.get_fastpath_enabled()
+    if mode == "int8":
+        torch.backends.mha.set_fastpath_enabled(False)
+    F.linear = routed
+    try:
+        with torch.no_grad():
+            h = stack(x, src_key_padding_mask=~alive)
+    finally:
+        F.linear = plain_linear
+        torch.backends.mha.set_fastpath_enabled(fast)
+    if mode == "int8" and hits[0] != 4 * n_layers:
+        raise AssertionError(f"{hits[0]} matmuls were diverted, expected {4 * n_layers}")
+    h = F.layer_norm(h, (d,), sd["norm_f.weight"], sd["norm_f.bias"], eps)
+    policy = plain_linear(h, sd["policy.weight"])
+    promo = plain_linear(h, sd["promo.weight"])
+    n = x.shape[0]
+    king = torch.where(control < 0, KING_BLACK, KING_WHITE).to(torch.int64)
+    raw = plain_linear(h[torch.arange(n), king], sd["value.weight"]).float()
+    if raw.shape[-1] == 1:
+        value = torch.tanh(raw).squeeze(-1)
+    else:
+        pr = torch.softmax(raw, dim=-1)
+        value = pr[:, 2] - pr[:, 0]
+    return policy, promo, value

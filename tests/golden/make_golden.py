@@ -1,0 +1,147 @@
+"""Writes tests/golden/reference_vectors.npz by running the reference's own Python.
+
+Run in the build container only (the reference tree is not present anywhere else):
+
+    python tests/golden/make_golden.py
+
+What it records, and why these need the reference itself rather than a closed form:
+
+* ``int8_linear`` (reference brokefish/nn/quant.py:281-305) on formula-generated inputs:
+  the true-division quantiser and the float64 sum over 256-wide k-chunks are not covered
+  by any vector the reference stores (its device tests use x * (1/s) and one chunk).
+* ``quantise_weights_int8_bytes`` / ``quantise_activations_int8`` (quant.py:246-278) on
+  the same inputs.
+* the end-to-end forward of ``BrokefishNet`` (brokefish/nn/model.py:621-645) in fp32 and
+  under ``emulated_forward(..., QuantConfig(fmt="int8"))`` (quant.py:498-506) on a net
+  whose weights are filled by the formula in :func:`fill_state_dict` (independent of any
+  RNG stream) and on eight build-defined positions, plus the layer-0 inputs of the first
+  patched matmul.
+
+Inputs are regenerated from the formulas below by the tests; only outputs are stored.
+"""
+from __future__ import annotations
+
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REFERENCE = "/root/reference"
+
+
+def formula(shape, a: int, b: int, mod: int, scale: float) -> torch.Tensor:
+    """Deterministic pseudo-random fp32 tensor: ((i*a + b) mod `mod` - mod//2) * scale."""
+    n = int(np.prod(shape))
+    i = np.arange(n, dtype=np.int64)
+    v = ((i * a + b) % mod - mod // 2).astype(np.float32) * np.float32(scale)
+    return torch.from_numpy(v.reshape(shape))
+
+
+def fill_state_dict(sd: dict) -> dict:
+    """Overwrite every floating tensor of a state_dict with formula values, distinct per
+    tensor and per layer; LayerNorm weights near one, biases small."""
+    out = {}
+    for k_idx, (name, t) in enumerate(sorted(sd.items())):
+        if not torch.is_floating_point(t):
+            out[name] = t.clone()
+            continue
+        fan = t.shape[-1] if t.dim() >= 2 else 1
+        if t.dim() == 2:
+            v = formula(t.shape, 7919 + 2 * k_idx, 104729 * (k_idx + 1), 2003, 1.0 / (1001.0 * fan ** 0.5) * 1.7)
+        elif name.endswith("norm1.weight") or name.endswith("norm2.weight") or name == "norm_f.weight":
+            v = 1.0 + formula(t.shape, 31 + k_idx, 17 * k_idx, 211, 0.002)
+        else:
+            v = formula(t.shape, 131 + k_idx, 29 * k_idx, 401, 0.0005)
+        out[name] = v.to(t.dtype)
+    return out
+
+
+# Eight build-defined positions: start, two openings with an en-passant flag and moved
+# pieces, captures with dead slots, a promoted queen in pawn slot 3, both sides to move,
+# a spread of clocks and repetition counts.
+def positions():
+    start = [8, 9, 10, 11, 12, 13, 14, 15, 65, 70, 130, 133, 192, 199, 259, 324,
+             1072, 1073, 1074, 1075, 1076, 1077, 1078, 1079, 1145, 1150, 1210, 1213, 1272, 1279, 1339, 1404]
+    b0 = list(start)
+    b1 = list(start); b1[4] = 28 | 0x200                       # e2e4, en-passant flag
+    b2 = list(b1); b2[4] = 28; b2[20] = 1024 | 36 | 0x200      # ... e7e5 flagged
+    b3 = list(b2); b3[20] = 0x800; b3[9] = 64 | 36; b3[4] = 28  # knight took e5, black pawn dead
+    b4 = list(b3); b4[3] = (4 << 6) | 59; b4[30] = 0x800        # promoted queen in pawn slot 3
+    b5 = list(b4); b5[15] = 320 | 0x200 | 6; b5[13] = 192 | 5   # white castled short (rook keeps special 0)
+    b6 = list(b5); b6[0] = 0x800; b6[1] = 0x800; b6[24] = 0x800; b6[31] = 1024 | 320 | 0x200 | 52
+    b7 = list(b6); b7[12] = 192 | 0x200 | 24
+    boards = np.array([b0, b1, b2, b3, b4, b5, b6, b7], dtype=np.uint16).view(np.int16)
+    control = np.array([1, -1, 1, -1, 37, -101, 100, -2], dtype=np.int16)
+    rep = np.array([0, 1, 2, 0, 1, 2, 0, 5], dtype=np.uint8)
+    return torch.from_numpy(boards), torch.from_numpy(control), torch.from_numpy(rep)
+
+
+def weight_checksum(q: np.ndarray) -> np.ndarray:
+    """Position-weighted int64 checksums of an int8 matrix (rows and columns)."""
+    q = q.astype(np.int64)
+    w = np.arange(q.size, dtype=np.int64).reshape(q.shape) % 1009 + 1
+    return np.array([(q * w).sum(), q.sum(), np.abs(q).sum(), (q[::3] * w[::3]).sum()], dtype=np.int64)
+
+
+def linear_cases():
+    """(name, x, w, bias, unsigned) for the standalone int8_linear vectors."""
+    cases = []
+    x1 = formula((32, 256), 31, 7, 401, 0.004) * (1.0 + 0.05 * torch.arange(32)[:, None])
+    w1 = formula((256, 256), 11, 5, 255, 0.0007)
+    cases.append(("s8_k256", x1, w1, formula((256,), 3, 1, 101, 0.01), False))
+    x2 = torch.relu(formula((32, 1024), 17, 3, 409, 0.003) * (1.0 + 0.03 * torch.arange(32)[:, None]))
+    w2 = formula((128, 1024), 13, 9, 251, 0.0009)
+    cases.append(("u8_k1024", x2, w2, formula((128,), 5, 2, 103, 0.02), True))
+    x3 = formula((16, 512), 29, 11, 397, 0.002)
+    w3 = formula((128, 512), 19, 4, 253, 0.0011)
+    cases.append(("s8_k512_nobias", x3, w3, None, False))
+    x4 = x1.clone(); x4[3] = 0.0                          # an all-zero row: scale must be 1
+    cases.append(("s8_zero_row", x4, w1, None, False))
+    return cases
+
+
+def main() -> int:
+    sys.path.insert(0, REFERENCE)
+    from brokefish.nn import quant as rq                      # noqa: E402
+    from brokefish.nn.model import BrokefishNet as RefNet     # noqa: E402
+
+    out = {}
+    for name, x, w, bias, unsigned in linear_cases():
+        y = rq.int8_linear(x, w, bias, unsigned=unsigned)
+        out[f"lin_{name}"] = y.numpy()
+        qb, ws = rq.quantise_weights_int8_bytes(w)
+        out[f"wqsum_{name}"] = weight_checksum(qb.view(torch.int8).numpy())
+        out[f"ws_{name}"] = ws.numpy()
+        q, s = rq.quantise_activations_int8(x[:, :256], unsigned)
+        out[f"qa_{name}"] = q.numpy().astype(np.int16)
+        out[f"sa_{name}"] = s.numpy()
+
+    for n_value in (1, 3):
+        torch.manual_seed(0)
+        net = RefNet(n_value=n_value).eval()
+        net.load_state_dict(fill_state_dict(net.state_dict()))
+        boards, control, rep = positions()
+        if n_value == 3:            # the second net only adds the value-head variant
+            boards, control, rep = boards[:3], control[:3], rep[:3]
+        captured = []
+        handle = net.encoder.layers[0].norm1.register_forward_hook(lambda m, i, o: captured.append(o.detach().clone()))
+        with torch.no_grad():
+            p32, q32, v32 = net(boards, control, rep)
+            handle.remove()
+            p8, q8, v8 = rq.emulated_forward(net, rq.QuantConfig(fmt="int8"))(boards, control, rep)
+        tag = f"nv{n_value}"
+        out[f"fp32_policy_{tag}"], out[f"fp32_promo_{tag}"], out[f"fp32_value_{tag}"] = p32.numpy(), q32.numpy(), v32.numpy()
+        out[f"int8_policy_{tag}"], out[f"int8_promo_{tag}"], out[f"int8_value_{tag}"] = p8.numpy(), q8.numpy(), v8.numpy()
+        if n_value == 1:
+            out["ln1_layer0"] = captured[0][:2].numpy()        # input of the first patched matmul, boards 0-1
+    out["torch_version"] = np.array(torch.__version__)
+    path = os.path.join(HERE, "reference_vectors.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, {k: getattr(v, "shape", None) for k, v in out.items()})
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

@@ -1,0 +1,149 @@
+"""Host-side logic that needs no GPU: the C-ABI surface, the weight packer, input checks."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import brokefish_amd
+from brokefish_amd import _build, hip_impl
+from brokefish_amd.net import BrokefishNet
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "brokefish_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    assert os.path.exists(_build.HIP_LIB), "build first: python -c 'import __graft_entry__ as g; g.build()'"
+    lib = ctypes.CDLL(_build.HIP_LIB)
+    names = _declared_functions()
+    assert {"bf_model_forward", "bf_wstream_bytes", "bf_fparams_floats", "bf_int8_q_max",
+            "bf_last_error", "bf_time_kernel_ms"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/brokefish_hip.h but not exported"
+
+
+def test_constants_agree_between_host_and_library():
+    # the counterpart of the reference's Python<->CUDA constant pin (tests/test_quant.py:233-269)
+    assert hip_impl.int8_q_max() == (hip_impl.Q_MAX_S8, hip_impl.Q_MAX_U8) == (127.0, 255.0)
+    lib = hip_impl.load_library()
+    shape = hip_impl._Shape(256, 8, 8, 1024, 1, 1e-5)
+    assert lib.bf_wstream_bytes(ctypes.byref(shape)) == (8 * 24 + 3) * 32768
+    bad = hip_impl._Shape(512, 16, 16, 2048, 1, 1e-5)
+    assert lib.bf_wstream_bytes(ctypes.byref(bad)) == 0 and lib.bf_fparams_floats(ctypes.byref(bad)) == 0
+
+
+def test_null_arguments_are_rejected_without_a_launch():
+    lib = hip_impl.load_library()
+    a = hip_impl._Args()
+    a.shape = hip_impl._Shape(256, 8, 8, 1024, 1, 1e-5)
+    a.n = 4
+    assert lib.bf_model_forward(ctypes.byref(a), None) == -1
+    assert b"must not be NULL" in lib.bf_last_error()
+    a.shape = hip_impl._Shape(512, 16, 16, 2048, 1, 1e-5)
+    assert lib.bf_model_forward(ctypes.byref(a), None) == -2
+    assert lib.bf_model_forward(None, None) == -1
+
+
+def test_packed_blocks_decode_back():
+    # re-derive the fragment index independently of the packer (the reference does the same for
+    # its own layout, tests/test_quant.py::test_the_packed_layout_decodes_back)
+    rng = np.random.default_rng(0)
+    wq = rng.integers(-127, 128, size=(768, 1024), dtype=np.int8)
+    blk = hip_impl.pack_int8_block(wq, n_tile=5, k0=512).view(np.int8)
+    assert blk.shape == (8, 64, 16)
+    for s, lane, r in [(0, 0, 0), (3, 17, 5), (7, 63, 15), (2, 40, 9), (5, 32, 0)]:
+        o, g = lane % 32, lane // 32
+        col = 512 + 32 * s + 8 * (r // 4) + 4 * g + (r % 4)
+        assert blk[s, lane, r] == wq[32 * 5 + o, col]
+    # every element of the 32 x 256 tile appears exactly once
+    tile = wq[160:192, 512:768]
+    assert sorted(blk.reshape(-1).tolist()) == sorted(tile.reshape(-1).tolist())
+    head = rng.standard_normal((96, 256)).astype(np.float32)
+    ht = hip_impl.pack_head_tile(head, 2)
+    assert ht.shape == (8, 4, 64, 4)
+    assert ht[3, 2, 45, 1] == head[64 + 13, 32 * 3 + 8 * 2 + 4 * 1 + 1]
+
+
+def test_pack_network_layout_and_sizes():
+    torch.manual_seed(0)
+    net = BrokefishNet(n_layers=2).eval().randomise_layers_()
+    sd = net.state_dict()
+    ws, fp = hip_impl.pack_network(sd, 2, 256, 1024, 1)
+    lib = hip_impl.load_library()
+    shape = hip_impl._Shape(256, 2, 8, 1024, 1, 1e-5)
+    assert ws.size == lib.bf_wstream_bytes(ctypes.byref(shape)) and ws.dtype == np.uint8
+    assert fp.size == lib.bf_fparams_floats(ctypes.byref(shape)) and fp.dtype == np.float32
+    layer_floats = (fp.size - (64 + 12 + 4 + 101 + 3 + 2) * 256) // 2
+    l1 = fp[layer_floats:2 * layer_floats]
+    assert (l1[:256] == sd["encoder.layers.1.norm1.weight"].numpy()).all()
+    assert (l1[512:1280] == sd["encoder.layers.1.self_attn.in_proj_bias"].numpy()).all()
+    q2, s2 = hip_impl.quantise_weights_int8(sd["encoder.layers.1.linear2.weight"])
+    wsum = l1[9 * 256 + 1024: 9 * 256 + 1024 + 4 * 256].view(np.int32).reshape(4, 256)
+    assert (wsum[2] == 128 * q2[:, 512:768].astype(np.int32).sum(1)).all()
+    sw = l1[9 * 256 + 1024 + 4 * 256:]
+    assert (sw[16:18] == s2).all()
+    assert (fp[2 * layer_floats:2 * layer_floats + 64 * 256] == sd["emb_square.weight"].numpy().reshape(-1)).all()
+    # second block of layer 0 is the K tile of head 0: rows 256..287 of in_proj
+    q_qkv, _ = hip_impl.quantise_weights_int8(sd["encoder.layers.0.self_attn.in_proj_weight"])
+    assert (ws[8192:16384].view(np.int8).reshape(8, 64, 16)[1, 35, 6] == q_qkv[256 + 3, 32 + 8 * 1 + 4 + 2])
+
+
+def test_registry_and_input_checks():
+    assert brokefish_amd.IMPLEMENTATIONS == ("hip",)
+    cls = brokefish_amd.encoder_impl("hip")
+    assert cls is hip_impl.FusedEncoder
+    with pytest.raises(ValueError):
+        brokefish_amd.encoder_impl("cuda")
+    chk = cls._check_inputs
+    b = torch.zeros(4, 32, dtype=torch.int16)
+    c = torch.ones(4, dtype=torch.int16)
+    r = torch.zeros(4, dtype=torch.uint8)
+    # the rejections the reference pins (tests/test_b2.py:325-343)
+    for bad in [(b.int(), c, r), (b[:, :31], c, r), (b, c.int(), r), (b, c[:3], r), (b, c, r.int()),
+                (b, c, r[:2]), (b.reshape(-1), c, r), (b[:0], c[:0], r[:0])]:
+        with pytest.raises(ValueError):
+            chk(*bad)
+    with pytest.raises(ValueError, match="GPU"):
+        chk(b, c, r)            # right types, wrong device
+    with pytest.raises(ValueError):
+        chk(b, c, r, mask=torch.zeros(4, 32, dtype=torch.int32))
+
+
+def test_constructor_rejections_do_not_need_a_gpu():
+    net = BrokefishNet(n_layers=1)
+    cls = hip_impl.FusedEncoder
+    with pytest.raises(NotImplementedError):
+        cls(net, fp8=True)
+    with pytest.raises(NotImplementedError):
+        cls(net, int8=False)
+    with pytest.raises(ValueError):
+        cls(net, acc_dtype="bf16")
+    with pytest.raises(ValueError):
+        cls(net.encoder, int8=True)                      # bare stack: forward_full needs the whole model
+    with pytest.raises(ValueError):
+        cls(BrokefishNet(d_model=128, n_heads=4, d_ff=512, n_layers=1), int8=True)
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="no GPU"):
+            cls(net, int8=True)
+
+
+def test_net_matches_reference_parameter_count_and_keys():
+    net = BrokefishNet()
+    assert sum(p.numel() for p in net.parameters()) == 6_383_360     # docs/reference/spec.md:328-331
+    keys = set(net.state_dict())
+    for k in ["emb_square.weight", "emb_type_special.weight", "emb_color_turn.weight", "emb_clock.weight",
+              "emb_rep.weight", "encoder.layers.7.self_attn.in_proj_weight", "encoder.layers.0.linear2.bias",
+              "encoder.layers.3.norm2.weight", "norm_f.bias", "policy.weight", "promo.weight", "value.weight"]:
+        assert k in keys
+    l0, l7 = net.encoder.layers[0], net.encoder.layers[7]
+    assert torch.equal(l0.linear1.weight, l7.linear1.weight)          # deep-copied layers at init
+    net.randomise_layers_()
+    assert not torch.equal(l0.linear1.weight, l7.linear1.weight)
