@@ -19,13 +19,17 @@ INCLUDE = os.path.join(ROOT, "include")
 HIP_LIB = os.path.join(HERE, "libbrokefish_hip.so")
 CHESSGEN_LIB = os.path.join(HERE, "libbf_chessgen.so")
 
-HIP_SOURCES = ["bf_eval.hip"]
+HIP_SOURCES = ["bf_host.hip", "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip"]
 # -ffp-contract=off: the kernel's fp32 arithmetic is specified operation by operation
 # (fused multiply-adds are written explicitly), so the compiler must not fuse on its own.
 # The packed-fp32 feature is disabled so no v_pk_*_f32 instructions are generated.
-HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
                "-ffp-contract=off", "-fno-fast-math",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               # the layer body is one fully unrolled straight-line block; the default
+               # unroll budgets would leave the last loops rolled and their register
+               # arrays in scratch memory
+               "-mllvm", "-pragma-unroll-threshold=10000000", "-mllvm", "-unroll-threshold=10000000",
                "-Wno-unused-command-line-argument"]
 
 
@@ -44,11 +48,24 @@ def _run(cmd):
 
 
 def build_hip(verbose: bool = False, extra=()) -> str:
-    srcs = [os.path.join(CSRC, s) for s in HIP_SOURCES]
-    cmd = [hipcc_path()] + HIPCC_FLAGS + list(extra) + ["-I", INCLUDE, "-I", CSRC, "-o", HIP_LIB] + srcs
-    r = _run(cmd)
-    if verbose:
-        print(r.stderr)
+    """Compile every translation unit (in parallel: the kernel variants take minutes each)
+    and link them into libbrokefish_hip.so."""
+    from concurrent.futures import ThreadPoolExecutor
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+
+    def compile_one(src):
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        cmd = [hipcc_path()] + HIPCC_FLAGS + list(extra) + ["-I", INCLUDE, "-I", CSRC, "-c",
+                                                            os.path.join(CSRC, src), "-o", obj]
+        r = _run(cmd)
+        if verbose:
+            print(r.stderr)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=len(HIP_SOURCES)) as pool:
+        objs = list(pool.map(compile_one, HIP_SOURCES))
+    _run([hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB] + objs)
     return HIP_LIB
 
 

@@ -1,0 +1,100 @@
+// Shared between the kernel translation units and the host side: layout constants and
+// the kernel argument block.  (Design notes follow.)
+//
+// Single-launch quantised network evaluator for gfx950 (MI355X).
+//
+// One wavefront evaluates one position: the 32 tokens of a board are the 32 columns of
+// every MFMA tile, and lanes l and l+32 share a token.  The residual stream
+// (32 tokens x 256 channels, fp32) lives in registers in MFMA accumulator layout for all
+// layers, so LayerNorm, the quantisers and the 32-token softmax are per-lane loops plus
+// one exchange with lane ^ 32.  All weight GEMMs are computed transposed,
+//     D[out_channel, token] = W[out_channel, k] * X^T[k, token]
+// with v_mfma_i32_32x32x32_i8, so a requantised output tile is already a valid B operand
+// of the next GEMM (the k order of an MFMA is free as long as both operands agree; the
+// host packs the weights in that order).  int8 weight tiles stream from HBM/L2 through a
+// double-buffered LDS ring with direct-to-LDS loads, 32 KiB per group, shared by the four
+// boards of a workgroup.  Attention (QK^T, PV) and the heads run on v_mfma_f32_32x32x2f32,
+// which accumulates as an exact chain of fused multiply-adds in k order.
+//
+// Arithmetic contract (what the CPU checker restates operation by operation):
+//   embedding  ((sq + ts) + ct) + (clock + rep)                        fp32
+//   LayerNorm  two partial sums per row (one per lane half), sequential over tiles then r
+//   quantise   s = amax / qmax, q = rint(x / s)  (x / s as a correctly rounded quotient)
+//   GEMM       exact int32; descale fl(fl(acc * sa) * sw) + b; several k-chunks are summed
+//              in fp64 before the single cast to fp32
+//   softmax    exp from bf_exp_neg, p * (1 / l)
+// See include/brokefish_hip.h for the blob layouts.
+
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "brokefish_hip.h"
+
+namespace bf {
+
+constexpr int T = 32;
+constexpr int THREADS = 256;
+constexpr int WAVES = 4;
+constexpr int FRAG = 1024;          // 64 lanes x 16 bytes
+constexpr int BLOCK = 8 * FRAG;     // one output tile over a 256-wide k-chunk
+constexpr int GROUP = 4 * BLOCK;    // unit of the LDS ring
+constexpr int RING = 2 * GROUP;
+
+constexpr int D = 256, F = 1024, NH = 8;
+constexpr int NT = D / 32;          // tiles across the model width
+constexpr int FT = F / 32;          // tiles across the FFN hidden width
+constexpr int KCF = F / 256;        // k-chunks of the second FFN matmul
+constexpr int LAYER_BLOCKS = 3 * NT + NT + FT + NT * KCF;
+constexpr int LAYER_GROUPS = LAYER_BLOCKS / 4;
+constexpr int HEAD_GROUPS = 3;
+static_assert(LAYER_BLOCKS % 8 == 0, "ring slot of a block must not depend on the layer");
+
+// per-layer side parameters, in floats
+constexpr int O_LN1G = 0, O_LN1B = D, O_BQKV = 2 * D, O_BOUT = 5 * D, O_LN2G = 6 * D,
+              O_LN2B = 7 * D, O_BFF1 = 8 * D, O_BFF2 = 8 * D + F, O_WSUM = 9 * D + F,
+              O_SW = 9 * D + F + KCF * D;
+constexpr int N_SW = 3 * D / 128 + D / 128 + F / 128 + D / 128;
+constexpr int LAYER_FLOATS = O_SW + ((N_SW + 3) / 4) * 4;
+// a layer's parameters are padded to a whole number of 4 KiB copies (one per workgroup pass)
+constexpr int PARAM_BYTES = ((LAYER_FLOATS * 4 + WAVES * FRAG - 1) / (WAVES * FRAG)) * (WAVES * FRAG);
+constexpr int PARAM_FLOATS = PARAM_BYTES / 4;
+constexpr int LDS_BYTES = RING + 2 * PARAM_BYTES;
+constexpr int SW_QKV = 0, SW_OUT = 3 * D / 128, SW_FF1 = SW_OUT + D / 128, SW_FF2 = SW_FF1 + F / 128;
+// global side parameters after the layers
+constexpr int G_SQ = 0, G_TS = 64 * D, G_CT = G_TS + 12 * D, G_CLOCK = G_CT + 4 * D,
+              G_REP = G_CLOCK + 101 * D, G_NFG = G_REP + 3 * D, G_NFB = G_NFG + D,
+              GLOBAL_FLOATS = G_NFB + D;
+
+constexpr int N_PHASES = 12;
+// phase slots of the optional cycle profile
+enum { PH_EMBED, PH_LN1, PH_QKV, PH_ATTN, PH_OUT, PH_LN2, PH_FF1, PH_FF2, PH_HEADS, PH_STORE, PH_SYNC, PH_TOTAL };
+
+struct KArgs {
+    const uint16_t* boards;
+    const int16_t* control;
+    const uint8_t* rep;
+    const uint64_t* mask;
+    int n;
+    const uint8_t* wstream;
+    const float* fparams;
+    void* policy;
+    void* promo;
+    float* value;
+    int* best;
+    int out_fp32, n_layers, l0, l1, n_value;
+    float eps;
+    float* xpark;                 // workspace: 32 KiB per board slot, residual stream parked during the FFN
+    unsigned long long* profile;  // [N_PHASES] cycle sums over waves, profile builds only
+    bf_taps taps;
+};
+
+// One launcher per separately compiled kernel variant (production, debug taps, phase
+// profile); each sets the dynamic-LDS limit once and launches on `stream`.
+hipError_t launch_prod(const KArgs& k, int grid, hipStream_t stream);
+hipError_t launch_taps(const KArgs& k, int grid, hipStream_t stream);
+hipError_t launch_prof(const KArgs& k, int grid, hipStream_t stream);
+
+}  // namespace bf

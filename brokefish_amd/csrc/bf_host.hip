@@ -1,0 +1,148 @@
+// Host side of the evaluator library: the C-ABI of include/brokefish_hip.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+
+#include "bf_args.h"
+
+
+
+static thread_local char g_err[512] = "";
+
+static int fail(int code, const char* msg) {
+    snprintf(g_err, sizeof(g_err), "%s", msg);
+    return code;
+}
+
+static bool shape_ok(const bf_shape* s) {
+    return s && s->d_model == bf::D && s->d_ff == bf::F && s->n_heads == bf::NH && s->n_layers >= 1 &&
+           (s->n_value == 1 || s->n_value == 3);
+}
+
+extern "C" size_t bf_wstream_bytes(const bf_shape* s) {
+    if (!shape_ok(s)) return 0;
+    return ((size_t)s->n_layers * bf::LAYER_GROUPS + bf::HEAD_GROUPS) * bf::GROUP;
+}
+
+extern "C" size_t bf_fparams_floats(const bf_shape* s) {
+    if (!shape_ok(s)) return 0;
+    return (size_t)s->n_layers * bf::PARAM_FLOATS + bf::GLOBAL_FLOATS;
+}
+
+extern "C" size_t bf_workspace_bytes(const bf_shape* s, int64_t n) {
+    if (!shape_ok(s) || n < 1) return 0;
+    const size_t slots = (size_t)((n + bf::WAVES - 1) / bf::WAVES) * bf::WAVES;
+    return slots * bf::T * bf::D * sizeof(float);
+}
+
+extern "C" size_t bf_layer_stride_floats(const bf_shape* s) {
+    if (!shape_ok(s)) return 0;
+    return bf::PARAM_FLOATS;
+}
+
+extern "C" void bf_int8_q_max(double* s8, double* u8) {
+    if (s8) *s8 = 127.0;
+    if (u8) *u8 = 255.0;
+}
+
+extern "C" const char* bf_last_error(void) { return g_err; }
+
+static int check_args(const bf_eval_args* a, bf::KArgs* k) {
+    if (!a) return fail(BF_ERR_ARGUMENT, "args is NULL");
+    if (!shape_ok(&a->shape))
+        return fail(BF_ERR_UNSUPPORTED,
+                    "unsupported network shape: this build carries d_model=256, n_heads=8, d_ff=1024, "
+                    "n_layers>=1, n_value in {1,3}");
+    if (a->n < 1 || a->n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
+    if (!a->boards || !a->control || !a->rep) return fail(BF_ERR_ARGUMENT, "boards/control/rep must not be NULL");
+    if (!a->wstream || !a->fparams) return fail(BF_ERR_ARGUMENT, "wstream/fparams must not be NULL");
+    if (!a->policy || !a->promo || !a->value) return fail(BF_ERR_ARGUMENT, "policy/promo/value must not be NULL");
+    if (((uintptr_t)a->wstream & 15) || ((uintptr_t)a->fparams & 15))
+        return fail(BF_ERR_ARGUMENT, "wstream/fparams must be 16-byte aligned");
+    if (((uintptr_t)a->policy & 15) || ((uintptr_t)a->promo & 7) || ((uintptr_t)a->boards & 1))
+        return fail(BF_ERR_ARGUMENT, "policy must be 16-byte and promo 8-byte aligned");
+    if (a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
+    if (!a->workspace || ((uintptr_t)a->workspace & 15) || a->workspace_bytes < bf_workspace_bytes(&a->shape, a->n))
+        return fail(BF_ERR_ARGUMENT, "workspace must be 16-byte aligned and hold bf_workspace_bytes(shape, n) bytes");
+    memset(k, 0, sizeof(*k));
+    k->boards = a->boards; k->control = a->control; k->rep = a->rep; k->mask = a->mask;
+    k->n = (int)a->n;
+    k->wstream = a->wstream; k->fparams = a->fparams;
+    k->policy = a->policy; k->promo = a->promo; k->value = a->value; k->best = a->best_move;
+    k->out_fp32 = a->out_fp32 ? 1 : 0;
+    k->xpark = static_cast<float*>(a->workspace);
+    k->n_layers = a->shape.n_layers; k->n_value = a->shape.n_value; k->eps = a->shape.eps;
+    k->l0 = 0; k->l1 = a->shape.n_layers;
+    if (a->taps) {
+        k->taps = *a->taps;
+        if (a->taps->layer_begin || a->taps->layer_end) {
+            k->l0 = a->taps->layer_begin; k->l1 = a->taps->layer_end;
+            if (k->l0 < 0 || k->l1 > k->n_layers || k->l0 > k->l1)
+                return fail(BF_ERR_ARGUMENT, "taps layer range must satisfy 0 <= begin <= end <= n_layers");
+        }
+        if (a->taps->x_in && ((uintptr_t)a->taps->x_in & 15)) return fail(BF_ERR_ARGUMENT, "x_in must be 16-byte aligned");
+    }
+    return BF_OK;
+}
+
+static int launch(const bf_eval_args* a, const bf::KArgs& k, hipStream_t stream) {
+    const int grid = (k.n + bf::WAVES - 1) / bf::WAVES;
+    const hipError_t e = k.profile ? bf::launch_prof(k, grid, stream)
+                       : a->taps   ? bf::launch_taps(k, grid, stream)
+                                   : bf::launch_prod(k, grid, stream);
+    if (e != hipSuccess) {
+        snprintf(g_err, sizeof(g_err), "kernel launch failed: %s", hipGetErrorString(e));
+        return BF_ERR_LAUNCH;
+    }
+    return BF_OK;
+}
+
+extern "C" int bf_model_forward(const bf_eval_args* args, void* stream) {
+    bf::KArgs k;
+    const int rc = check_args(args, &k);
+    if (rc) return rc;
+    return launch(args, k, (hipStream_t)stream);
+}
+
+extern "C" int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_t* cycles) {
+    bf::KArgs k;
+    const int rc = check_args(args, &k);
+    if (rc) return rc;
+    if (args->taps) return fail(BF_ERR_ARGUMENT, "the phase profile runs without taps");
+    if (!cycles) return fail(BF_ERR_ARGUMENT, "cycles must not be NULL");
+    k.profile = reinterpret_cast<unsigned long long*>(cycles);
+    return launch(args, k, (hipStream_t)stream);
+}
+
+extern "C" int bf_profile_phase_count(void) { return bf::N_PHASES; }
+
+extern "C" const char* bf_profile_phase_name(int i) {
+    static const char* names[bf::N_PHASES] = {"embed", "ln1_quant", "qkv_gemm_epilogue", "attention",
+                                              "oquant_outproj", "ln2_quant", "ffn1", "ffn2", "heads",
+                                              "store", "ring_wait", "total"};
+    return (i >= 0 && i < bf::N_PHASES) ? names[i] : "";
+}
+
+extern "C" double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int iters) {
+    bf::KArgs k;
+    int rc = check_args(args, &k);
+    if (rc) return rc;
+    if (iters < 1 || warmup < 0) return fail(BF_ERR_ARGUMENT, "iters must be >= 1 and warmup >= 0");
+    hipStream_t s = (hipStream_t)stream;
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+        return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    for (int i = 0; i < warmup && !rc; i++) rc = launch(args, k, s);
+    (void)hipEventRecord(e0, s);
+    for (int i = 0; i < iters && !rc; i++) rc = launch(args, k, s);
+    (void)hipEventRecord(e1, s);
+    const hipError_t e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc) return rc;
+    if (e != hipSuccess) return fail(BF_ERR_LAUNCH, hipGetErrorString(e));
+    return (double)ms / iters;
+}

@@ -1,36 +1,12 @@
-// Single-launch quantised network evaluator for gfx950 (MI355X).
-//
-// One wavefront evaluates one position: the 32 tokens of a board are the 32 columns of
-// every MFMA tile, and lanes l and l+32 share a token.  The residual stream
-// (32 tokens x 256 channels, fp32) lives in registers in MFMA accumulator layout for all
-// layers, so LayerNorm, the quantisers and the 32-token softmax are per-lane loops plus
-// one exchange with lane ^ 32.  All weight GEMMs are computed transposed,
-//     D[out_channel, token] = W[out_channel, k] * X^T[k, token]
-// with v_mfma_i32_32x32x32_i8, so a requantised output tile is already a valid B operand
-// of the next GEMM (the k order of an MFMA is free as long as both operands agree; the
-// host packs the weights in that order).  int8 weight tiles stream from HBM/L2 through a
-// double-buffered LDS ring with direct-to-LDS loads, 32 KiB per group, shared by the four
-// boards of a workgroup.  Attention (QK^T, PV) and the heads run on v_mfma_f32_32x32x2f32,
-// which accumulates as an exact chain of fused multiply-adds in k order.
-//
-// Arithmetic contract (what the CPU checker restates operation by operation):
-//   embedding  ((sq + ts) + ct) + (clock + rep)                        fp32
-//   LayerNorm  two partial sums per row (one per lane half), sequential over tiles then r
-//   quantise   s = amax / qmax, q = rint(x / s)  (x / s as a correctly rounded quotient)
-//   GEMM       exact int32; descale fl(fl(acc * sa) * sw) + b; several k-chunks are summed
-//              in fp64 before the single cast to fp32
-//   softmax    exp from bf_exp_neg, p * (1 / l)
-// See include/brokefish_hip.h for the blob layouts.
+// Device code of the evaluator (see bf_args.h for the design notes).  Included by one
+// translation unit per kernel variant so the variants compile in parallel.
+#pragma once
 
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
-#include <cstdio>
-#include <cstring>
+#include "bf_args.h"
 
-#include "brokefish_hip.h"
-
-typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -39,51 +15,6 @@ typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
 namespace bf {
 
-constexpr int T = 32;
-constexpr int THREADS = 256;
-constexpr int WAVES = 4;
-constexpr int FRAG = 1024;          // 64 lanes x 16 bytes
-constexpr int BLOCK = 8 * FRAG;     // one output tile over a 256-wide k-chunk
-constexpr int GROUP = 4 * BLOCK;    // unit of the LDS ring
-constexpr int RING = 2 * GROUP;
-
-constexpr int D = 256, F = 1024, NH = 8;
-constexpr int NT = D / 32;          // tiles across the model width
-constexpr int FT = F / 32;          // tiles across the FFN hidden width
-constexpr int KCF = F / 256;        // k-chunks of the second FFN matmul
-constexpr int LAYER_BLOCKS = 3 * NT + NT + FT + NT * KCF;
-constexpr int LAYER_GROUPS = LAYER_BLOCKS / 4;
-constexpr int HEAD_GROUPS = 3;
-static_assert(LAYER_BLOCKS % 8 == 0, "ring slot of a block must not depend on the layer");
-
-// per-layer side parameters, in floats
-constexpr int O_LN1G = 0, O_LN1B = D, O_BQKV = 2 * D, O_BOUT = 5 * D, O_LN2G = 6 * D,
-              O_LN2B = 7 * D, O_BFF1 = 8 * D, O_BFF2 = 8 * D + F, O_WSUM = 9 * D + F,
-              O_SW = 9 * D + F + KCF * D;
-constexpr int N_SW = 3 * D / 128 + D / 128 + F / 128 + D / 128;
-constexpr int LAYER_FLOATS = O_SW + ((N_SW + 3) / 4) * 4;
-constexpr int SW_QKV = 0, SW_OUT = 3 * D / 128, SW_FF1 = SW_OUT + D / 128, SW_FF2 = SW_FF1 + F / 128;
-// global side parameters after the layers
-constexpr int G_SQ = 0, G_TS = 64 * D, G_CT = G_TS + 12 * D, G_CLOCK = G_CT + 4 * D,
-              G_REP = G_CLOCK + 101 * D, G_NFG = G_REP + 3 * D, G_NFB = G_NFG + D,
-              GLOBAL_FLOATS = G_NFB + D;
-
-struct KArgs {
-    const uint16_t* boards;
-    const int16_t* control;
-    const uint8_t* rep;
-    const uint64_t* mask;
-    int n;
-    const uint8_t* wstream;
-    const float* fparams;
-    void* policy;
-    void* promo;
-    float* value;
-    int* best;
-    int out_fp32, n_layers, l0, l1, n_value;
-    float eps;
-    bf_taps taps;
-};
 
 __device__ __forceinline__ constexpr int ch(int r, int g) { return 8 * (r / 4) + 4 * g + (r % 4); }
 
@@ -121,14 +52,36 @@ __device__ __forceinline__ float tanh_dev(float x) {
     return __builtin_copysignf(th, x);
 }
 
+// Program-order anchors: an empty volatile asm that reads and writes a register forces the
+// value to exist at this point, so the compiler cannot postpone a tile's epilogue past the
+// following tiles (which would keep every accumulator alive and spill it).
+__device__ __forceinline__ void pin(float& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void pin(double& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void pin(int& v) { asm volatile("" : "+v"(v)); }
+
+__device__ __forceinline__ void pin16(float (&v)[16]) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) pin(v[i]);
+}
+
 __device__ __forceinline__ v4f ldg4(const float* p) { return *reinterpret_cast<const v4f*>(p); }
 __device__ __forceinline__ v4i ldg4i(const float* p) { return *reinterpret_cast<const v4i*>(p); }
+// the 16 per-channel parameters a lane needs for one 32-wide tile starting at p
+__device__ __forceinline__ void load_tile16(const float* p, int g, v4f (&b)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) b[j] = ldg4(p + 8 * j + 4 * g);
+}
+__device__ __forceinline__ void load_tile16i(const float* p, int g, v4i (&b)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) b[j] = ldg4i(p + 8 * j + 4 * g);
+}
 
-extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];
+extern __shared__ __attribute__((aligned(1024))) uint8_t ring[];   // ring, then two parameter buffers
 
 // ---- LDS ring ----------------------------------------------------------------------
 
 struct Stream {
+    unsigned long long t_sync;  // cycles spent waiting in ring_sync (profile builds only)
     const uint8_t* base;  // wstream
     int pos;              // next position (in consumption order) to issue
     int body_groups;      // groups of the layers that run
@@ -137,8 +90,11 @@ struct Stream {
     int total;            // positions in this launch
 };
 
+template <bool GUARDED>
 __device__ __forceinline__ void issue_group(Stream& st, int wave, int lane) {
-    if (st.pos < st.total) {
+    // Inside the layers the next position always exists (the head tiles follow), so the
+    // unguarded form keeps the layer body free of branches.
+    if (!GUARDED || st.pos < st.total) {
         const int gid = st.pos < st.body_groups ? st.first_gid + st.pos
                                                 : st.head_gid + (st.pos - st.body_groups);
         const uint8_t* src = st.base + (size_t)gid * GROUP + (size_t)wave * BLOCK + lane * 16;
@@ -152,34 +108,68 @@ __device__ __forceinline__ void issue_group(Stream& st, int wave, int lane) {
     st.pos++;
 }
 
-// Called before the first block of every group: this group's bytes have landed, every
-// wave is done with the previous group, so its half of the ring can be refilled.
-__device__ __forceinline__ void ring_sync(Stream& st, int wave, int lane) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    issue_group(st, wave, lane);
+// One layer's side parameters (PARAM_BYTES) into parameter buffer `buf`.
+__device__ __forceinline__ void issue_params(const float* fparams, int layer, int buf, int wave, int lane) {
+    const uint8_t* src = reinterpret_cast<const uint8_t*>(fparams) + (size_t)layer * PARAM_BYTES + wave * FRAG + lane * 16;
+    uint8_t* dst = ring + RING + buf * PARAM_BYTES + wave * FRAG;
+#pragma unroll
+    for (int i = 0; i < PARAM_BYTES / (WAVES * FRAG); i++)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(src + i * WAVES * FRAG),
+            (__attribute__((address_space(3))) void*)(dst + i * WAVES * FRAG), 16, 0, 0);
 }
 
-#define BF_BLOCK(blk)                                  \
-    ([&]() -> int {                                    \
-        if (((blk) & 3) == 0) ring_sync(st, wave, lane); \
-        return ((blk) & 7) * BLOCK;                    \
-    }())
+// Called before the first block of a group is read from LDS: this group's bytes have
+// landed, every wave has finished reading the previous group (its fragment reads have
+// returned), so that half of the ring can be refilled.
+template <bool GUARDED, bool PROF = false>
+__device__ __forceinline__ void ring_sync(Stream& st, int wave, int lane) {
+    unsigned long long t0 = 0;
+    if (PROF) t0 = __builtin_readcyclecounter();
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (PROF) st.t_sync += __builtin_readcyclecounter() - t0;
+    issue_group<GUARDED>(st, wave, lane);
+}
+
+// Fragments of block `blk` (index within the layer; LAYER_BLOCKS = block 0 of the next layer).
+template <bool PROF>
+__device__ __forceinline__ void load_frags(int blk, v4i (&fr)[8], Stream& st, int wave, int lane) {
+    if ((blk & 3) == 0) ring_sync<false, PROF>(st, wave, lane);
+    const int off = (blk & 7) * BLOCK;
+#pragma unroll
+    for (int s = 0; s < 8; s++) fr[s] = *reinterpret_cast<const v4i*>(&ring[off + s * FRAG + lane * 16]);
+}
 
 // acc[out_channel r][token] (weights as A) or acc[token r][out_channel] (SWAP, weights as B)
 template <bool SWAP>
-__device__ __forceinline__ v16i gemm_tile(int off, const v4i (&act)[8], int lane) {
+__device__ __forceinline__ v16i mfma8(const v4i (&w)[8], const v4i (&act)[8]) {
     v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int s = 0; s < 8; s++) {
-        const v4i w = *reinterpret_cast<const v4i*>(&ring[off + s * FRAG + lane * 16]);
-        acc = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act[s], w, acc, 0, 0, 0)
-                   : __builtin_amdgcn_mfma_i32_32x32x32_i8(w, act[s], acc, 0, 0, 0);
-    }
+    for (int s = 0; s < 8; s++)
+        acc = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act[s], w[s], acc, 0, 0, 0)
+                   : __builtin_amdgcn_mfma_i32_32x32x32_i8(w[s], act[s], acc, 0, 0, 0);
     return acc;
 }
 
 // ---- row operations -------------------------------------------------------------------
+
+// four quotients v / sa (correctly rounded) -> round to nearest even -> low bytes packed
+__device__ __forceinline__ unsigned quant4(float v0, float v1, float v2, float v3, float sa, float inv) {
+    unsigned w = 0;
+    const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        // correctly rounded v / sa from the reciprocal and two fused corrections
+        const float q0 = v[i] * inv;
+        const float rem = __builtin_fmaf(-q0, sa, v[i]);
+        const float qf = __builtin_fmaf(rem, inv, q0);
+        // adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low bits
+        const unsigned m = (unsigned)__float_as_int(qf + 12582912.0f);
+        w |= (m & 0xffu) << (8 * i);
+    }
+    return w;
+}
 
 // signed int8 quantiser of one token row spread over two lanes; y is [tiles][16]
 template <int NTILES>
@@ -195,24 +185,11 @@ __device__ __forceinline__ void quant_s8(const float (&y)[NTILES][16], int g, v4
 #pragma unroll
     for (int n = 0; n < NTILES; n++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            unsigned w = 0;
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float v = y[n][4 * j + i];
-                // correctly rounded v / sa from the reciprocal and two fused corrections
-                const float q0 = v * inv;
-                const float rem = __builtin_fmaf(-q0, sa, v);
-                const float qf = __builtin_fmaf(rem, inv, q0);
-                // adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low bits
-                const unsigned m = (unsigned)__float_as_int(qf + 12582912.0f);
-                w |= (m & 0xffu) << (8 * i);
-            }
-            q[n][j] = (int)w;
-        }
+        for (int j = 0; j < 4; j++)
+            q[n][j] = (int)quant4(y[n][4 * j], y[n][4 * j + 1], y[n][4 * j + 2], y[n][4 * j + 3], sa, inv);
 }
 
-// LayerNorm of the residual rows, affine applied, in the fixed lane order
+// LayerNorm of the residual rows, affine applied, in the fixed lane order; gamma/beta in LDS or global
 __device__ __forceinline__ void layernorm(const float (&x)[NT][16], const float* gamma, const float* beta,
                                           float eps, int g, float (&y)[NT][16]) {
     float s = 0.0f;
@@ -247,8 +224,24 @@ __device__ __forceinline__ void layernorm(const float (&x)[NT][16], const float*
 
 // ---- the kernel ------------------------------------------------------------------------
 
-template <bool TAPS>
+template <bool TAPS, bool PROF>
 __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
+    unsigned long long ph[N_PHASES];
+    unsigned long long t_mark = 0, t_begin = 0;
+    if (PROF) {
+#pragma unroll
+        for (int i = 0; i < N_PHASES; i++) ph[i] = 0;
+        t_mark = t_begin = __builtin_readcyclecounter();
+    }
+    // close the current phase: everything since the last mark is charged to `slot`
+#define BF_PHASE(slot)                                              \
+    do {                                                            \
+        if (PROF) {                                                 \
+            const unsigned long long now_ = __builtin_readcyclecounter(); \
+            ph[slot] += now_ - t_mark;                              \
+            t_mark = now_;                                          \
+        }                                                           \
+    } while (0)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t = lane & 31, g = lane >> 5;
@@ -257,15 +250,17 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
     const int b = valid ? board_raw : a.n - 1;  // idle waves shadow the last board, store nothing
 
     Stream st;
+    st.t_sync = 0;
     st.base = a.wstream;
     st.pos = 0;
     st.body_groups = (a.l1 - a.l0) * LAYER_GROUPS;
     st.first_gid = a.l0 * LAYER_GROUPS;
     st.head_gid = a.n_layers * LAYER_GROUPS;
     st.total = st.body_groups + HEAD_GROUPS;
-    issue_group(st, wave, lane);
+    issue_group<true>(st, wave, lane);
+    if (a.l0 < a.l1) issue_params(a.fparams, a.l0, 0, wave, lane);
 
-    const float* gp = a.fparams + (size_t)a.n_layers * LAYER_FLOATS;
+    const float* gp = a.fparams + (size_t)a.n_layers * PARAM_FLOATS;
 
     // ---- embedding ---------------------------------------------------------------------
     float x[NT][16];
@@ -320,10 +315,24 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
     }
 
     // ---- layers --------------------------------------------------------------------------
+    // `fr` always holds the weight fragments of the next block to be multiplied: each
+    // block's MFMA chain is followed at once by the LDS reads of the block after it.
+    v4i fr[8];
+    BF_PHASE(PH_EMBED);
+    if (a.l0 < a.l1) load_frags<PROF>(0, fr, st, wave, lane);
     const int nl_run = a.l1 - a.l0;
     for (int l = a.l0; l < a.l1; l++) {
-        const float* lp = a.fparams + (size_t)l * LAYER_FLOATS;
-        const size_t bl = (size_t)b * nl_run + (l - a.l0);  // tap row
+        const int li = l - a.l0;
+        const float* lp = reinterpret_cast<const float*>(&ring[RING + (li & 1) * PARAM_BYTES]);
+        const size_t bl = (size_t)b * nl_run + li;  // tap row
+        const bool more = l + 1 < a.l1;
+        // multiply by the block in `fr`, then fetch the fragments of the block after it
+#define BF_MM(SWAP, blk, act)                                                   \
+    ([&]() -> v16i {                                                            \
+        const v16i r_ = mfma8<SWAP>(fr, act);                                   \
+        if ((blk) + 1 < LAYER_BLOCKS || more) load_frags<PROF>((blk) + 1, fr, st, wave, lane); \
+        return r_;                                                              \
+    }())
 
         v4i xq[NT];
         float sa;
@@ -339,6 +348,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                 for (int j = 0; j < 4; j++)
                     *reinterpret_cast<int*>(a.taps.qa_qkv + (bl * T + t) * D + 32 * n + 8 * j + 4 * g) = xq[n][j];
         }
+        BF_PHASE(PH_LN1);
         // activation scale of token ch(r, g), for the V tiles whose rows are tokens
         float sa_tok[16];
 #pragma unroll
@@ -348,49 +358,40 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         float o[NH][16];
 #pragma unroll
         for (int h = 0; h < NH; h++) {
+            // parameters of this head's three tiles, fetched ahead of the matrix products
+            const float swq = lp[O_SW + SW_QKV + (32 * h) / 128];
+            const float swk = lp[O_SW + SW_QKV + (D + 32 * h) / 128];
+            const float swv = lp[O_SW + SW_QKV + (2 * D + 32 * h) / 128];
+            const float bv = lp[O_BQKV + 2 * D + 32 * h + t];
+            v4f bq[4], bk[4];
+            load_tile16(lp + O_BQKV + 32 * h, g, bq);
+            load_tile16(lp + O_BQKV + D + 32 * h, g, bk);
+            const v16i accq = BF_MM(false, 3 * h + 0, xq);
+            const v16i acck = BF_MM(false, 3 * h + 1, xq);
+            const v16i accv = BF_MM(true, 3 * h + 2, xq);   // V transposed: lane = channel, registers = tokens
+            // The next layer's parameters can be fetched once every wave is inside this layer
+            // (after the last layer the same layer is fetched again, into the idle buffer).
+            if (h == 1) issue_params(a.fparams, more ? l + 1 : l, (li + 1) & 1, wave, lane);
             float qf[16], kf[16], vf[16];
             {
-                const v16i acc = gemm_tile<false>(BF_BLOCK(3 * h + 0), xq, lane);
-                const float sw = lp[O_SW + SW_QKV + (32 * h) / 128];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v4f bi = ldg4(lp + O_BQKV + 32 * h + 8 * j + 4 * g);
+                for (int j = 0; j < 4; j++)
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        qf[4 * j + i] = ((float)acc[4 * j + i] * sa) * sw + bi[i];
-                }
+                    for (int i = 0; i < 4; i++) {
+                        qf[4 * j + i] = ((float)accq[4 * j + i] * sa) * swq + bq[j][i];
+                        kf[4 * j + i] = ((float)acck[4 * j + i] * sa) * swk + bk[j][i];
+                    }
+#pragma unroll
+                for (int r = 0; r < 16; r++) vf[r] = ((float)accv[r] * sa_tok[r]) * swv + bv;
                 if (TAPS && a.taps.acc_qkv && valid)
 #pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        a.taps.acc_qkv[(bl * T + t) * 3 * D + 32 * h + ch(r, g)] = acc[r];
+                    for (int r = 0; r < 16; r++) {
+                        a.taps.acc_qkv[(bl * T + t) * 3 * D + 32 * h + ch(r, g)] = accq[r];
+                        a.taps.acc_qkv[(bl * T + t) * 3 * D + D + 32 * h + ch(r, g)] = acck[r];
+                        a.taps.acc_qkv[(bl * T + ch(r, g)) * 3 * D + 2 * D + 32 * h + t] = accv[r];
+                    }
             }
-            {
-                const v16i acc = gemm_tile<false>(BF_BLOCK(3 * h + 1), xq, lane);
-                const float sw = lp[O_SW + SW_QKV + (D + 32 * h) / 128];
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v4f bi = ldg4(lp + O_BQKV + D + 32 * h + 8 * j + 4 * g);
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        kf[4 * j + i] = ((float)acc[4 * j + i] * sa) * sw + bi[i];
-                }
-                if (TAPS && a.taps.acc_qkv && valid)
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        a.taps.acc_qkv[(bl * T + t) * 3 * D + D + 32 * h + ch(r, g)] = acc[r];
-            }
-            {
-                // V tile transposed: lane = channel, registers = tokens
-                const v16i acc = gemm_tile<true>(BF_BLOCK(3 * h + 2), xq, lane);
-                const float sw = lp[O_SW + SW_QKV + (2 * D + 32 * h) / 128];
-                const float bi = lp[O_BQKV + 2 * D + 32 * h + t];
-#pragma unroll
-                for (int r = 0; r < 16; r++) vf[r] = ((float)acc[r] * sa_tok[r]) * sw + bi;
-                if (TAPS && a.taps.acc_qkv && valid)
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        a.taps.acc_qkv[(bl * T + ch(r, g)) * 3 * D + 2 * D + 32 * h + t] = acc[r];
-            }
+            BF_PHASE(PH_QKV);
             // scores, transposed: lane = query token, register r = key ch(r, g)
             v16f sc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -417,6 +418,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
             for (int r = 0; r < 16; r++) oa = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[r], p[r] * rl, oa, 0, 0, 0);
 #pragma unroll
             for (int r = 0; r < 16; r++) o[h][r] = oa[r];
+            BF_PHASE(PH_ATTN);
         }
 
         // ---- output projection + residual -------------------------------------------------
@@ -431,30 +433,53 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                     for (int j = 0; j < 4; j++)
                         *reinterpret_cast<int*>(a.taps.qa_out + (bl * T + t) * D + 32 * n + 8 * j + 4 * g) = oq[n][j];
             }
+            v16i acc2[2];
+            acc2[0] = BF_MM(false, 3 * NT, oq);
+            v4f bcur[4];
+            load_tile16(lp + O_BOUT, g, bcur);
 #pragma unroll
             for (int n = 0; n < NT; n++) {
-                const v16i acc = gemm_tile<false>(BF_BLOCK(3 * NT + n), oq, lane);
+                if (n + 1 < NT) acc2[(n + 1) & 1] = BF_MM(false, 3 * NT + n + 1, oq);
+                v4f bnxt[4];   // parameters are fetched one tile ahead of their use
+                if (n + 1 < NT) load_tile16(lp + O_BOUT + 32 * (n + 1), g, bnxt);
+                const v16i acc = acc2[n & 1];
                 const float sw = lp[O_SW + SW_OUT + (32 * n) / 128];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v4f bi = ldg4(lp + O_BOUT + 32 * n + 8 * j + 4 * g);
+                for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int i = 0; i < 4; i++)
-                        x[n][4 * j + i] = x[n][4 * j + i] + (((float)acc[4 * j + i] * so) * sw + bi[i]);
-                }
+                        x[n][4 * j + i] = x[n][4 * j + i] + (((float)acc[4 * j + i] * so) * sw + bcur[j][i]);
+                pin16(x[n]);
                 if (TAPS && a.taps.acc_out && valid)
 #pragma unroll
                     for (int r = 0; r < 16; r++)
                         a.taps.acc_out[(bl * T + t) * D + 32 * n + ch(r, g)] = acc[r];
+#pragma unroll
+                for (int j = 0; j < 4; j++) bcur[j] = bnxt[j];
             }
         }
 
+        BF_PHASE(PH_OUT);
         // ---- feed-forward ------------------------------------------------------------------
         {
             float y[NT][16];
             layernorm(x, lp + O_LN2G, lp + O_LN2B, a.eps, g, y);
             quant_s8<NT>(y, g, xq, sa);
         }
+        // The residual stream is not needed again until the second FFN matmul's epilogue:
+        // park it in the workspace (one coalesced 1 KiB store per register quad) so that
+        // the hidden activations have the register file to themselves.
+        {
+            float* xp = a.xpark + (size_t)board_raw * (T * D) + lane * 4;
+#pragma unroll
+            for (int n = 0; n < NT; n++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const v4f v = {x[n][4 * j], x[n][4 * j + 1], x[n][4 * j + 2], x[n][4 * j + 3]};
+                    *reinterpret_cast<v4f*>(xp + (n * 4 + j) * 256) = v;
+                }
+        }
+        BF_PHASE(PH_LN2);
         if (TAPS && a.taps.qa_ff1 && valid) {
 #pragma unroll
             for (int n = 0; n < NT; n++)
@@ -464,85 +489,115 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         }
         v4i hq[KCF][8];
         float sh[KCF];
-#pragma unroll
-        for (int c = 0; c < KCF; c++) {
+        {
+            v16i acc2[2];
+            acc2[0] = BF_MM(false, 4 * NT, xq);
             float hf[8][16];
             float am = 0.0f;
+            v4f bcur[4];
+            load_tile16(lp + O_BFF1, g, bcur);
 #pragma unroll
-            for (int s = 0; s < 8; s++) {
-                const int tile = 8 * c + s;
-                const v16i acc = gemm_tile<false>(BF_BLOCK(4 * NT + tile), xq, lane);
+            for (int tile = 0; tile < FT; tile++) {
+                const int c = tile / 8, s = tile % 8;
+                if (tile + 1 < FT) acc2[(tile + 1) & 1] = BF_MM(false, 4 * NT + tile + 1, xq);
+                v4f bnxt[4];
+                if (tile + 1 < FT) load_tile16(lp + O_BFF1 + 32 * (tile + 1), g, bnxt);
+                const v16i acc = acc2[tile & 1];
                 const float sw = lp[O_SW + SW_FF1 + (32 * tile) / 128];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v4f bi = ldg4(lp + O_BFF1 + 32 * tile + 8 * j + 4 * g);
+                for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const float v = __builtin_fmaxf(((float)acc[4 * j + i] * sa) * sw + bi[i], 0.0f);
+                        const float v = __builtin_fmaxf(((float)acc[4 * j + i] * sa) * sw + bcur[j][i], 0.0f);
                         hf[s][4 * j + i] = v;
                         am = __builtin_fmaxf(am, v);
                     }
-                }
+                pin16(hf[s]);
+#pragma unroll
+                for (int j = 0; j < 4; j++) bcur[j] = bnxt[j];
                 if (TAPS && a.taps.acc_ff1 && valid)
 #pragma unroll
                     for (int r = 0; r < 16; r++)
                         a.taps.acc_ff1[(bl * T + t) * F + 32 * tile + ch(r, g)] = acc[r];
-            }
-            // unsigned quantiser over this 256-wide chunk; bytes stored as q - 128 for the
-            // signed MFMA, the offset is added back through wsum
-            am = __builtin_fmaxf(am, partner(am, g));
-            const float s8 = am > 0.0f ? am / 255.0f : 1.0f;
-            const float inv = 1.0f / s8;
-            sh[c] = s8;
+                if (s == 7) {
+                    // unsigned quantiser over this 256-wide chunk; bytes stored as q - 128 for
+                    // the signed MFMA, the offset is added back through wsum
+                    am = __builtin_fmaxf(am, partner(am, g));
+                    const float s8 = am > 0.0f ? am / 255.0f : 1.0f;
+                    const float inv = 1.0f / s8;
+                    sh[c] = s8;
 #pragma unroll
-            for (int s = 0; s < 8; s++)
+                    for (int s2 = 0; s2 < 8; s2++)
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const unsigned w = quant4(hf[s2][4 * j], hf[s2][4 * j + 1], hf[s2][4 * j + 2],
+                                                      hf[s2][4 * j + 3], s8, inv);
+                            if (TAPS && a.taps.qa_ff2 && valid)
+                                *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 256 * c + 32 * s2 + 8 * j + 4 * g) = w;
+                            hq[c][s2][j] = (int)(w ^ 0x80808080u);
+                        }
+                    am = 0.0f;
+                }
+            }
+        }
+        BF_PHASE(PH_FF1);
+        {
+            const float* xp = a.xpark + (size_t)board_raw * (T * D) + lane * 4;
+#pragma unroll
+            for (int n = 0; n < NT; n++)
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    unsigned w = 0;
+                    const v4f v = *reinterpret_cast<const v4f*>(xp + (n * 4 + j) * 256);
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const float v = hf[s][4 * j + i];
-                        const float q0 = v * inv;
-                        const float rem = __builtin_fmaf(-q0, s8, v);
-                        const float qf = __builtin_fmaf(rem, inv, q0);
-                        const unsigned m = (unsigned)__float_as_int(qf + 12582912.0f);
-                        w |= (m & 0xffu) << (8 * i);
-                    }
-                    if (TAPS && a.taps.qa_ff2 && valid)
-                        *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 256 * c + 32 * s + 8 * j + 4 * g) = w;
-                    hq[c][s][j] = (int)(w ^ 0x80808080u);
+                    for (int i = 0; i < 4; i++) x[n][4 * j + i] = v[i];
                 }
         }
-#pragma unroll
-        for (int n = 0; n < NT; n++) {
+        {
+            v16i acc2[2];
+            acc2[0] = BF_MM(false, 4 * NT + FT, hq[0]);
             double o64[16];
+            v4i wcur[4];
+            load_tile16i(lp + O_WSUM, g, wcur);
+            v4f bout[4];
 #pragma unroll
-            for (int c = 0; c < KCF; c++) {
-                const v16i acc = gemm_tile<false>(BF_BLOCK(4 * NT + FT + n * KCF + c), hq[c], lane);
+            for (int idx = 0; idx < NT * KCF; idx++) {
+                const int n = idx / KCF, c = idx % KCF;
+                if (idx + 1 < NT * KCF) acc2[(idx + 1) & 1] = BF_MM(false, 4 * NT + FT + idx + 1, hq[(idx + 1) % KCF]);
+                v4i wnxt[4];
+                if (idx + 1 < NT * KCF)
+                    load_tile16i(lp + O_WSUM + ((idx + 1) % KCF) * D + 32 * ((idx + 1) / KCF), g, wnxt);
+                if (c == 0) load_tile16(lp + O_BFF2 + 32 * n, g, bout);   // used three blocks later
+                const v16i acc = acc2[idx & 1];
                 const double sc = (double)sh[c];
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v4i ws = ldg4i(lp + O_WSUM + c * D + 32 * n + 8 * j + 4 * g);
+                for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const int full = acc[4 * j + i] + ws[i];
+                        const int full = acc[4 * j + i] + wcur[j][i];
                         // exact product, one rounding in the add: same as out += acc * sa in fp64
                         o64[4 * j + i] = c == 0 ? (double)full * sc
                                                 : __builtin_fma((double)full, sc, o64[4 * j + i]);
                         if (TAPS && a.taps.acc_ff2 && valid)
                             a.taps.acc_ff2[((bl * KCF + c) * T + t) * D + 32 * n + 8 * j + 4 * g + i] = full;
                     }
+                if (c == KCF - 1) {
+                    const float sw = lp[O_SW + SW_FF2 + (32 * n) / 128];
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            x[n][4 * j + i] = x[n][4 * j + i] + ((float)o64[4 * j + i] * sw + bout[j][i]);
+                    pin16(x[n]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) pin(o64[i]);
                 }
-            }
-            const float sw = lp[O_SW + SW_FF2 + (32 * n) / 128];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const v4f bi = ldg4(lp + O_BFF2 + 32 * n + 8 * j + 4 * g);
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-                    x[n][4 * j + i] = x[n][4 * j + i] + ((float)o64[4 * j + i] * sw + bi[i]);
+                for (int j = 0; j < 4; j++) wcur[j] = wnxt[j];
             }
         }
+#undef BF_MM
+        BF_PHASE(PH_FF2);
         if (TAPS && a.taps.resid && valid) {
 #pragma unroll
             for (int n = 0; n < NT; n++)
@@ -566,7 +621,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
 #pragma unroll
     for (int m = 0; m < 3; m++) {
         // one 32 KiB group per head tile
-        ring_sync(st, wave, lane);
+        ring_sync<true, PROF>(st, wave, lane);
         const int off = (m & 1) * GROUP;
         v16f acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -580,6 +635,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
             }
         head[m] = acc;
     }
+    BF_PHASE(PH_HEADS);
     // Nothing may leave before every wave has finished with the ring (no further sync follows).
     if (!valid) return;
 
@@ -645,116 +701,30 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         }
         if (lane == 0) a.best[b] = bi == 0x7fffffff ? -1 : bi;
     }
+    if (PROF) {
+        BF_PHASE(PH_STORE);
+        ph[PH_SYNC] = st.t_sync;
+        ph[PH_TOTAL] = __builtin_readcyclecounter() - t_begin;
+        if (lane == 0 && a.profile)
+#pragma unroll
+            for (int i = 0; i < N_PHASES; i++) atomicAdd(&a.profile[i], ph[i]);
+    }
+#undef BF_PHASE
+}
+
+
+template <bool TAPS, bool PROF>
+hipError_t launch_variant(const KArgs& k, int grid, hipStream_t stream) {
+    // more than 64 KiB of dynamic LDS has to be requested once per kernel (per thread: cheap)
+    static thread_local bool lds_set = false;
+    if (!lds_set) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&eval_kernel<TAPS, PROF>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+        if (e != hipSuccess) return e;
+        lds_set = true;
+    }
+    hipLaunchKernelGGL((eval_kernel<TAPS, PROF>), dim3(grid), dim3(THREADS), LDS_BYTES, stream, k);
+    return hipGetLastError();
 }
 
 }  // namespace bf
-
-// ---- host side --------------------------------------------------------------------------------
-
-static thread_local char g_err[512] = "";
-
-static int fail(int code, const char* msg) {
-    snprintf(g_err, sizeof(g_err), "%s", msg);
-    return code;
-}
-
-static bool shape_ok(const bf_shape* s) {
-    return s && s->d_model == bf::D && s->d_ff == bf::F && s->n_heads == bf::NH && s->n_layers >= 1 &&
-           (s->n_value == 1 || s->n_value == 3);
-}
-
-extern "C" size_t bf_wstream_bytes(const bf_shape* s) {
-    if (!shape_ok(s)) return 0;
-    return ((size_t)s->n_layers * bf::LAYER_GROUPS + bf::HEAD_GROUPS) * bf::GROUP;
-}
-
-extern "C" size_t bf_fparams_floats(const bf_shape* s) {
-    if (!shape_ok(s)) return 0;
-    return (size_t)s->n_layers * bf::LAYER_FLOATS + bf::GLOBAL_FLOATS;
-}
-
-extern "C" void bf_int8_q_max(double* s8, double* u8) {
-    if (s8) *s8 = 127.0;
-    if (u8) *u8 = 255.0;
-}
-
-extern "C" const char* bf_last_error(void) { return g_err; }
-
-static int check_args(const bf_eval_args* a, bf::KArgs* k) {
-    if (!a) return fail(BF_ERR_ARGUMENT, "args is NULL");
-    if (!shape_ok(&a->shape))
-        return fail(BF_ERR_UNSUPPORTED,
-                    "unsupported network shape: this build carries d_model=256, n_heads=8, d_ff=1024, "
-                    "n_layers>=1, n_value in {1,3}");
-    if (a->n < 1 || a->n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
-    if (!a->boards || !a->control || !a->rep) return fail(BF_ERR_ARGUMENT, "boards/control/rep must not be NULL");
-    if (!a->wstream || !a->fparams) return fail(BF_ERR_ARGUMENT, "wstream/fparams must not be NULL");
-    if (!a->policy || !a->promo || !a->value) return fail(BF_ERR_ARGUMENT, "policy/promo/value must not be NULL");
-    if (((uintptr_t)a->wstream & 15) || ((uintptr_t)a->fparams & 15))
-        return fail(BF_ERR_ARGUMENT, "wstream/fparams must be 16-byte aligned");
-    if (((uintptr_t)a->policy & 15) || ((uintptr_t)a->promo & 7) || ((uintptr_t)a->boards & 1))
-        return fail(BF_ERR_ARGUMENT, "policy must be 16-byte and promo 8-byte aligned");
-    if (a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
-    memset(k, 0, sizeof(*k));
-    k->boards = a->boards; k->control = a->control; k->rep = a->rep; k->mask = a->mask;
-    k->n = (int)a->n;
-    k->wstream = a->wstream; k->fparams = a->fparams;
-    k->policy = a->policy; k->promo = a->promo; k->value = a->value; k->best = a->best_move;
-    k->out_fp32 = a->out_fp32 ? 1 : 0;
-    k->n_layers = a->shape.n_layers; k->n_value = a->shape.n_value; k->eps = a->shape.eps;
-    k->l0 = 0; k->l1 = a->shape.n_layers;
-    if (a->taps) {
-        k->taps = *a->taps;
-        if (a->taps->layer_begin || a->taps->layer_end) {
-            k->l0 = a->taps->layer_begin; k->l1 = a->taps->layer_end;
-            if (k->l0 < 0 || k->l1 > k->n_layers || k->l0 > k->l1)
-                return fail(BF_ERR_ARGUMENT, "taps layer range must satisfy 0 <= begin <= end <= n_layers");
-        }
-        if (a->taps->x_in && ((uintptr_t)a->taps->x_in & 15)) return fail(BF_ERR_ARGUMENT, "x_in must be 16-byte aligned");
-    }
-    return BF_OK;
-}
-
-static int launch(const bf_eval_args* a, const bf::KArgs& k, hipStream_t stream) {
-    const int grid = (k.n + bf::WAVES - 1) / bf::WAVES;
-    if (a->taps)
-        hipLaunchKernelGGL(bf::eval_kernel<true>, dim3(grid), dim3(bf::THREADS), bf::RING, stream, k);
-    else
-        hipLaunchKernelGGL(bf::eval_kernel<false>, dim3(grid), dim3(bf::THREADS), bf::RING, stream, k);
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) {
-        snprintf(g_err, sizeof(g_err), "kernel launch failed: %s", hipGetErrorString(e));
-        return BF_ERR_LAUNCH;
-    }
-    return BF_OK;
-}
-
-extern "C" int bf_model_forward(const bf_eval_args* args, void* stream) {
-    bf::KArgs k;
-    const int rc = check_args(args, &k);
-    if (rc) return rc;
-    return launch(args, k, (hipStream_t)stream);
-}
-
-extern "C" double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int iters) {
-    bf::KArgs k;
-    int rc = check_args(args, &k);
-    if (rc) return rc;
-    if (iters < 1 || warmup < 0) return fail(BF_ERR_ARGUMENT, "iters must be >= 1 and warmup >= 0");
-    hipStream_t s = (hipStream_t)stream;
-    hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
-        return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
-    for (int i = 0; i < warmup && !rc; i++) rc = launch(args, k, s);
-    hipEventRecord(e0, s);
-    for (int i = 0; i < iters && !rc; i++) rc = launch(args, k, s);
-    hipEventRecord(e1, s);
-    const hipError_t e = hipEventSynchronize(e1);
-    float ms = 0.0f;
-    hipEventElapsedTime(&ms, e0, e1);
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
-    if (rc) return rc;
-    if (e != hipSuccess) return fail(BF_ERR_LAUNCH, hipGetErrorString(e));
-    return (double)ms / iters;
-}

@@ -1,0 +1,6 @@
+// Kernel variant "prod" of the evaluator, compiled as its own translation unit.
+#include "bf_kernel.hip.h"
+
+namespace bf {
+hipError_t launch_prod(const KArgs& k, int grid, hipStream_t stream) { return launch_variant<false, false>(k, grid, stream); }
+}  // namespace bf

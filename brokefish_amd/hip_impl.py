@@ -53,7 +53,8 @@ class _Args(C.Structure):
                 ("mask", C.c_void_p), ("n", C.c_int64), ("shape", _Shape),
                 ("wstream", C.c_void_p), ("fparams", C.c_void_p),
                 ("policy", C.c_void_p), ("promo", C.c_void_p), ("value", C.c_void_p),
-                ("best_move", C.c_void_p), ("out_fp32", C.c_int32), ("taps", C.POINTER(_Taps))]
+                ("best_move", C.c_void_p), ("out_fp32", C.c_int32),
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("taps", C.POINTER(_Taps))]
 
 
 _lib = None
@@ -78,6 +79,15 @@ def load_library():
         L.bf_wstream_bytes.argtypes = [C.POINTER(_Shape)]
         L.bf_fparams_floats.restype = C.c_size_t
         L.bf_fparams_floats.argtypes = [C.POINTER(_Shape)]
+        L.bf_workspace_bytes.restype = C.c_size_t
+        L.bf_workspace_bytes.argtypes = [C.POINTER(_Shape), C.c_int64]
+        L.bf_layer_stride_floats.restype = C.c_size_t
+        L.bf_layer_stride_floats.argtypes = [C.POINTER(_Shape)]
+        L.bf_profile_phases.restype = C.c_int
+        L.bf_profile_phases.argtypes = [C.POINTER(_Args), C.c_void_p, C.c_void_p]
+        L.bf_profile_phase_count.restype = C.c_int
+        L.bf_profile_phase_name.restype = C.c_char_p
+        L.bf_profile_phase_name.argtypes = [C.c_int]
         L.bf_int8_q_max.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_double)]
         _lib = L
     return _lib
@@ -136,9 +146,16 @@ def pack_head_tile(head: np.ndarray, m: int) -> np.ndarray:
     return np.ascontiguousarray(head[rows, cols], dtype=np.float32)
 
 
-def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_value: int):
+def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_value: int,
+                 layer_stride: Optional[int] = None):
     """state_dict -> (wstream uint8 [bytes], fparams float32 [floats]) in the layouts of
-    include/brokefish_hip.h."""
+    include/brokefish_hip.h.  ``layer_stride`` is the per-layer stride of fparams in floats
+    (default: what the library reports for this shape)."""
+    if layer_stride is None:
+        shape = _Shape(d, n_layers, d // 32, f, n_value, 1e-5)
+        layer_stride = int(load_library().bf_layer_stride_floats(C.byref(shape)))
+        if not layer_stride:
+            raise ValueError("the library has no kernel for this shape")
     nt, ft, kcf = d // 32, f // 32, f // 256
     get = lambda k: sd[k].detach().float().cpu()
     stream, fl = [], []
@@ -161,11 +178,15 @@ def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_v
         wsum = (128 * q_ff2.astype(np.int32).reshape(d, kcf, 256).sum(axis=2)).T   # [kcf, d]
         sw = np.concatenate([s_qkv, s_out, s_ff1, s_ff2]).astype(np.float32)
         sw = np.concatenate([sw, np.zeros((-len(sw)) % 4, np.float32)])
-        fl += [get(p + "norm1.weight").numpy(), get(p + "norm1.bias").numpy(),
-               get(p + "self_attn.in_proj_bias").numpy(), get(p + "self_attn.out_proj.bias").numpy(),
-               get(p + "norm2.weight").numpy(), get(p + "norm2.bias").numpy(),
-               get(p + "linear1.bias").numpy(), get(p + "linear2.bias").numpy(),
-               np.ascontiguousarray(wsum, dtype=np.int32).view(np.float32).reshape(-1), sw]
+        layer = [get(p + "norm1.weight").numpy(), get(p + "norm1.bias").numpy(),
+                 get(p + "self_attn.in_proj_bias").numpy(), get(p + "self_attn.out_proj.bias").numpy(),
+                 get(p + "norm2.weight").numpy(), get(p + "norm2.bias").numpy(),
+                 get(p + "linear1.bias").numpy(), get(p + "linear2.bias").numpy(),
+                 np.ascontiguousarray(wsum, dtype=np.int32).view(np.float32).reshape(-1), sw]
+        used = sum(x.size for x in layer)
+        if used > layer_stride:
+            raise ValueError("layer parameters do not fit the library's layer stride")
+        fl += layer + [np.zeros(layer_stride - used, np.float32)]
     head = np.zeros((96, d), np.float32)
     head[:N_POLICY] = get("policy.weight").numpy()
     head[N_POLICY:N_POLICY + N_PROMO] = get("promo.weight").numpy()
@@ -270,6 +291,8 @@ class FusedEncoder:
             self.promo_out = torch.empty(n, T, N_PROMO, device=self.device, dtype=self.out_dtype)
             self.value_out = torch.empty(n, device=self.device, dtype=torch.float32)
             self.best_out = torch.empty(n, device=self.device, dtype=torch.int32)
+            nbytes = self._lib.bf_workspace_bytes(C.byref(self._shape), n)
+            self.workspace = torch.empty(nbytes, device=self.device, dtype=torch.uint8)
             self._buffered_full = n
 
     @staticmethod
@@ -302,6 +325,10 @@ class FusedEncoder:
         a.policy, a.promo, a.value = policy.data_ptr(), promo.data_ptr(), value.data_ptr()
         a.best_move = best.data_ptr() if (best is not None and mask is not None) else None
         a.out_fp32 = 1 if policy.dtype is torch.float32 else 0
+        need = self._lib.bf_workspace_bytes(C.byref(self._shape), a.n)
+        if getattr(self, "workspace", None) is None or self.workspace.numel() < need:
+            self.workspace = torch.empty(need, device=self.device, dtype=torch.uint8)
+        a.workspace, a.workspace_bytes = self.workspace.data_ptr(), self.workspace.numel()
         a.taps = C.pointer(taps) if taps is not None else None
         return a
 
@@ -345,6 +372,24 @@ class FusedEncoder:
         if ms < 0:
             raise RuntimeError(f"bf_time_kernel_ms failed ({ms}): {self._lib.bf_last_error().decode()}")
         return ms
+
+    def profile_phases(self, boards, control, rep, mask=None) -> Dict[str, float]:
+        """Shader-clock cycles per phase, averaged over the wavefronts of one launch (the
+        counterpart of the reference's read_profile / profile_phases)."""
+        n = self._check_inputs(boards, control, rep, mask)
+        self._ensure_full_buffers(n)
+        k = self._lib.bf_profile_phase_count()
+        cyc = torch.zeros(k, dtype=torch.int64, device=self.device)
+        args = self._args(boards.contiguous(), control.contiguous(), rep.contiguous(),
+                          mask.contiguous() if mask is not None else None,
+                          self.policy_out, self.promo_out, self.value_out, self.best_out)
+        rc = self._lib.bf_profile_phases(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
+                                         C.c_void_p(cyc.data_ptr()))
+        if rc:
+            raise RuntimeError(f"bf_profile_phases failed ({rc}): {self._lib.bf_last_error().decode()}")
+        torch.cuda.current_stream(self.device).synchronize()
+        waves = 4 * ((n + 3) // 4)
+        return {self._lib.bf_profile_phase_name(i).decode(): cyc[i].item() / waves for i in range(k)}
 
     # -- debug taps (the counterpart of the reference's forward_stage) ------------
 

@@ -46,6 +46,12 @@ typedef struct {
  * the end of this header).  Return 0 for an unsupported shape. */
 size_t bf_wstream_bytes(const bf_shape* s);   /* int8 weight tiles + fp32 head tiles */
 size_t bf_fparams_floats(const bf_shape* s);  /* fp32 / int32 side parameters        */
+size_t bf_layer_stride_floats(const bf_shape* s); /* stride of one layer inside fparams */
+/* Device scratch the caller lends to a launch of n positions (32 KiB per position, rounded
+ * up to a whole workgroup): the kernel parks the fp32 residual stream there while the
+ * feed-forward hidden activations occupy the register file.  Contents are meaningless
+ * between launches; launches that may overlap need separate workspaces. */
+size_t bf_workspace_bytes(const bf_shape* s, int64_t n);
 
 /* Optional debug outputs ("taps") and teacher forcing.  All pointers may be NULL.
  * B = boards in the call, L = layers run, kc = K / 256.
@@ -92,6 +98,8 @@ typedef struct {
     float* value;
     int32_t* best_move;
     int32_t out_fp32;
+    void* workspace;        /* bf_workspace_bytes(shape, n) bytes of device memory */
+    size_t workspace_bytes;
     const bf_taps* taps; /* NULL in production */
 } bf_eval_args;
 
@@ -114,6 +122,18 @@ const char* bf_last_error(void);
  * (reference csrc/encoder.cu:1886-1903) at whole-kernel granularity. */
 double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int iters);
 
+/* In-kernel phase accounting, the counterpart of the reference's profile hooks
+ * (reference csrc/encoder.cu:1083-1177 and :1886-1903: set_profile / read_profile /
+ * profile_phases).  bf_profile_phases runs a separately compiled build of the evaluator
+ * that reads the shader clock at phase boundaries and adds, per wavefront, the cycles of
+ * each phase into cycles[bf_profile_phase_count()] (DEVICE memory, caller-zeroed).  Slot
+ * "ring_wait" is the time spent waiting for weight tiles at LDS-ring synchronisations and
+ * is also contained in the enclosing phases; slot "total" is the wavefront lifetime.
+ * The production kernel carries none of this code. */
+int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_t* cycles);
+int bf_profile_phase_count(void);
+const char* bf_profile_phase_name(int i);
+
 /* -------------------------------------------------------------------------------------
  * Blob layouts (what the host packer writes; brokefish_amd/hip_impl.py is the packer).
  *
@@ -132,7 +152,9 @@ double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int
  * of [policy(64); promo(4); value(n_value); zeros]), fragment (n, q), lane 32g + o holds
  * the four floats W[32 m + o][32 n + 8 q + 4 g + 0..3].
  *
- * fparams (fp32 unless noted), per layer at stride bf_layer_floats:
+ * fparams (fp32 unless noted), per layer at stride bf_layer_stride_floats() (the layer's
+ * parameters zero-padded to a multiple of 4 KiB, because a workgroup copies them to LDS
+ * in 4 KiB passes):
  *     ln1_gamma[d] ln1_beta[d] b_qkv[3d] b_out[d] ln2_gamma[d] ln2_beta[d] b_ffn1[f]
  *     b_ffn2[d] wsum[kc_f][d] (int32: 128 * sum of the int8 weights of ffn2 row over
  *     k-chunk c) sw_qkv[3d/128] sw_out[d/128] sw_ffn1[f/128] sw_ffn2[d/128]

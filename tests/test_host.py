@@ -25,7 +25,8 @@ def test_library_loads_and_exports_every_declared_symbol():
     lib = ctypes.CDLL(_build.HIP_LIB)
     names = _declared_functions()
     assert {"bf_model_forward", "bf_wstream_bytes", "bf_fparams_floats", "bf_int8_q_max",
-            "bf_last_error", "bf_time_kernel_ms"} <= set(names)
+            "bf_last_error", "bf_time_kernel_ms", "bf_layer_stride_floats", "bf_workspace_bytes",
+            "bf_profile_phases", "bf_profile_phase_count", "bf_profile_phase_name"} <= set(names)
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in include/brokefish_hip.h but not exported"
 
@@ -36,6 +37,8 @@ def test_constants_agree_between_host_and_library():
     lib = hip_impl.load_library()
     shape = hip_impl._Shape(256, 8, 8, 1024, 1, 1e-5)
     assert lib.bf_wstream_bytes(ctypes.byref(shape)) == (8 * 24 + 3) * 32768
+    assert lib.bf_workspace_bytes(ctypes.byref(shape), 4096) == 4096 * 32768
+    assert lib.bf_workspace_bytes(ctypes.byref(shape), 5) == 8 * 32768
     bad = hip_impl._Shape(512, 16, 16, 2048, 1, 1e-5)
     assert lib.bf_wstream_bytes(ctypes.byref(bad)) == 0 and lib.bf_fparams_floats(ctypes.byref(bad)) == 0
 
@@ -82,13 +85,15 @@ def test_pack_network_layout_and_sizes():
     assert ws.size == lib.bf_wstream_bytes(ctypes.byref(shape)) and ws.dtype == np.uint8
     assert fp.size == lib.bf_fparams_floats(ctypes.byref(shape)) and fp.dtype == np.float32
     layer_floats = (fp.size - (64 + 12 + 4 + 101 + 3 + 2) * 256) // 2
+    assert layer_floats == lib.bf_layer_stride_floats(ctypes.byref(shape)) and layer_floats % 1024 == 0
     l1 = fp[layer_floats:2 * layer_floats]
     assert (l1[:256] == sd["encoder.layers.1.norm1.weight"].numpy()).all()
     assert (l1[512:1280] == sd["encoder.layers.1.self_attn.in_proj_bias"].numpy()).all()
     q2, s2 = hip_impl.quantise_weights_int8(sd["encoder.layers.1.linear2.weight"])
     wsum = l1[9 * 256 + 1024: 9 * 256 + 1024 + 4 * 256].view(np.int32).reshape(4, 256)
     assert (wsum[2] == 128 * q2[:, 512:768].astype(np.int32).sum(1)).all()
-    sw = l1[9 * 256 + 1024 + 4 * 256:]
+    sw = l1[9 * 256 + 1024 + 4 * 256:9 * 256 + 1024 + 4 * 256 + 20]
+    assert (l1[9 * 256 + 1024 + 4 * 256 + 20:] == 0).all()
     assert (sw[16:18] == s2).all()
     assert (fp[2 * layer_floats:2 * layer_floats + 64 * 256] == sd["emb_square.weight"].numpy().reshape(-1)).all()
     # second block of layer 0 is the K tile of head 0: rows 256..287 of in_proj
