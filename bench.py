@@ -59,6 +59,11 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=4096)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=64)
+    ap.add_argument("--sweep", action="store_true",
+                    help="also time batch sizes 64..65536 (per-launch latency regime) and add them to the line")
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run one device copy of this many MiB (a kernel of known HBM traffic, "
+                         "to calibrate FETCH_SIZE / WRITE_SIZE counter runs)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this path runs on one GPU (positions shard with no exchange step); --gpus must be 1",
@@ -75,6 +80,12 @@ def main() -> int:
     b, c, r, m = positions.random_positions(a.batch, plies=120, seed=0)
     bd, cd, rd, md = b.cuda(), c.cuda(), r.cuda(), m.cuda()
 
+    if a.copy_probe_mib:
+        src = torch.empty(a.copy_probe_mib << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(a.warmup):
         model.forward_full(bd, cd, rd, md)
     torch.cuda.synchronize()
@@ -100,6 +111,15 @@ def main() -> int:
                      "frac": achieved / (PEAK_INT8_OPS / 1e12), "traffic": None,
                      "kernel_ms": kern_ms, "ops_per_launch": OPS_PER_EVAL * a.batch},
     }
+    if a.sweep:
+        # the batch-size sweep of the small-batch latency regime: same net, same generator
+        pts = []
+        for nb in (64, 256, 1024, 4096, 16384, 65536):
+            sb, sc, sr, sm = (t.cuda() for t in positions.random_positions(nb, plies=120, seed=0))
+            ms = model.time_kernel_ms(sb, sc, sr, sm, warmup=3, iters=20)
+            pts.append({"batch": nb, "ms_per_launch": ms, "evals_per_s": nb / ms * 1e3})
+            del sb, sc, sr, sm
+        line["sweep"] = pts
     if not a.no_cpu:
         threads = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
         line["cpu_baseline"] = cpu_baseline(net, a.cpu_batch, threads)

@@ -64,7 +64,7 @@ def load_library():
     """The C-ABI library, loaded once.  Raises if it has not been built."""
     global _lib
     if _lib is None:
-        path = _build.HIP_LIB
+        path = os.environ.get("BROKEFISH_HIP_LIB", _build.HIP_LIB)   # override: A/B of two builds
         if not os.path.exists(path):
             raise RuntimeError(
                 f"{path} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
@@ -232,14 +232,16 @@ class FusedEncoder:
                 "all four matmuls of every layer are int8 here, which is the reference's 'all' scheme")
         if out_dtype not in (torch.float16, torch.float32):
             raise ValueError(f"out_dtype must be float16 or float32, got {out_dtype}")
-        if not hasattr(source, "encoder") or not hasattr(source, "policy"):
-            raise ValueError("forward_full needs the whole model: build this from a BrokefishNet "
-                             "(embeddings, encoder, norm_f and heads), not from a bare encoder stack")
-        if getattr(source, "value_head", "king") != "king" or getattr(source, "reinject", "none") != "none" \
-                or getattr(source, "rule_features", False):
+        # Like the reference class, this is built either from the whole network (boards in,
+        # logits out) or from a bare pre-norm encoder stack (the backbone call only).
+        net = source if hasattr(source, "encoder") and hasattr(source, "policy") else None
+        if net is None and not hasattr(source, "layers"):
+            raise ValueError("source must be a BrokefishNet or an nn.TransformerEncoder stack")
+        if net is not None and (getattr(net, "value_head", "king") != "king"
+                                or getattr(net, "reinject", "none") != "none"
+                                or getattr(net, "rule_features", False)):
             raise NotImplementedError("only the king value head without re-injection or rule features")
-        net = source
-        layers = net.encoder.layers
+        layers = (net.encoder if net is not None else source).layers
         first = layers[0]
         self.n_layers = len(layers)
         self.d_model = first.self_attn.embed_dim
@@ -253,7 +255,7 @@ class FusedEncoder:
                 f"got {self.d_model}, {self.d_ff}, {self.n_heads}")
         if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
             raise ValueError("the evaluator implements pre-norm ReLU layers only")
-        self.n_value = int(net.value.weight.shape[0])
+        self.n_value = int(net.value.weight.shape[0]) if net is not None else 1
         if self.n_value not in (1, 3):
             raise ValueError(f"value head must have 1 or 3 rows, got {self.n_value}")
         self.acc_dtype, self.fp8, self.int8 = acc_dtype, False, True
@@ -269,7 +271,15 @@ class FusedEncoder:
             raise RuntimeError("no GPU visible: the evaluator has no CPU path")
         self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
         self._shape = _Shape(self.d_model, self.n_layers, self.n_heads, self.d_ff, self.n_value, self.eps)
-        sd = {k: v.detach() for k, v in net.state_dict().items()}
+        if net is not None:
+            sd = {k: v.detach() for k, v in net.state_dict().items()}
+        else:   # bare stack: inert tables, identity final norm, zero heads (never read back)
+            d = self.d_model
+            sd = {"encoder." + k: v.detach() for k, v in source.state_dict().items()}
+            for name, rows in (("emb_square", 64), ("emb_type_special", 12), ("emb_color_turn", 4),
+                               ("emb_clock", 101), ("emb_rep", 3), ("policy", 64), ("promo", 4), ("value", 1)):
+                sd[name + ".weight"] = torch.zeros(rows, d)
+            sd["norm_f.weight"], sd["norm_f.bias"] = torch.ones(d), torch.zeros(d)
         wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value)
         if wstream.size != self._lib.bf_wstream_bytes(C.byref(self._shape)) or \
                 fparams.size != self._lib.bf_fparams_floats(C.byref(self._shape)):
@@ -339,6 +349,44 @@ class FusedEncoder:
 
     # -- the call ----------------------------------------------------------------
 
+    def _require_net(self, what: str):
+        if self.net is None:
+            raise ValueError(f"{what} needs the whole model: build this from a BrokefishNet, not "
+                             "from a bare nn.TransformerEncoder")
+        return self.net
+
+    def forward(self, x, alive=None, out=None):
+        """The encoder stack alone (reference brokefish/nn/cuda_impl.py:447-463):
+        ``x [n, 32, d]`` tokens and ``alive [n, 32]`` (bool or int8; dead tokens are masked
+        out of attention as keys) to the residual stream after the last layer, in ``x``'s
+        dtype.  The arithmetic inside is the same fp32 / int8 path as ``forward_full``.
+        """
+        n, t, d = x.shape
+        if d != self.d_model or t != T:
+            raise ValueError(f"expected [n, {T}, {self.d_model}], got {tuple(x.shape)}")
+        if not x.is_cuda:
+            raise ValueError("x must be on the GPU")
+        if alive is None:
+            alive_b = torch.ones(n, t, dtype=torch.bool, device=x.device)
+        else:
+            if alive.shape != (n, t):
+                raise ValueError(f"alive must be [{n}, {t}], got {tuple(alive.shape)}")
+            if alive.dtype not in (torch.bool, torch.int8):
+                raise ValueError(f"alive must be bool or int8, got {alive.dtype}")
+            alive_b = alive.bool()
+        # a captured slot is the word 0x800; only that bit reaches the attention mask here
+        boards = torch.where(alive_b, 0, 0x800).to(torch.int16)
+        control = torch.ones(n, dtype=torch.int16, device=x.device)
+        rep = torch.zeros(n, dtype=torch.uint8, device=x.device)
+        res = self.forward_taps(boards, control, rep, x_in=x.float().contiguous(), want=["resid"])
+        y = res["resid"][:, -1].to(x.dtype)
+        if out is not None:
+            out.copy_(y)
+            return out
+        return y
+
+    __call__ = forward
+
     def forward_full(self, boards, control, rep, mask=None):
         """Boards to ``(policy_logits, promo, value)`` in one launch.
 
@@ -346,6 +394,7 @@ class FusedEncoder:
         ``mask`` illegal entries are ``-inf`` and ``self.best_move`` ([n] int32) is the
         masked argmax.  Returns views on internal buffers, which the next call overwrites.
         """
+        self._require_net("forward_full")
         n = self._check_inputs(boards, control, rep, mask)
         self._ensure_full_buffers(n)
         boards, control, rep = boards.contiguous(), control.contiguous(), rep.contiguous()

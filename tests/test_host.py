@@ -132,7 +132,7 @@ def test_constructor_rejections_do_not_need_a_gpu():
     with pytest.raises(ValueError):
         cls(net, acc_dtype="bf16")
     with pytest.raises(ValueError):
-        cls(net.encoder, int8=True)                      # bare stack: forward_full needs the whole model
+        cls(object(), int8=True)                         # neither a network nor an encoder stack
     with pytest.raises(ValueError):
         cls(BrokefishNet(d_model=128, n_heads=4, d_ff=512, n_layers=1), int8=True)
     if not torch.cuda.is_available():

@@ -225,6 +225,29 @@ def test_teacher_forced_layers_against_the_torch_restatement(nets):
     assert (got["value"].cpu() - ref[2]).abs().max() < 1e-5
 
 
+def test_backbone_call_from_a_bare_encoder_stack(nets):
+    # reference brokefish/nn/cuda_impl.py:447-463 and tests/test_model.py: the stack alone, x in, x out
+    net, sd, model, co = nets["distinct"]
+    bare = encoder_impl("hip")(net.encoder, int8=True)
+    with pytest.raises(ValueError):
+        bare.forward_full(*_dev(*positions.random_positions(2, plies=4, seed=1, with_mask=False)))
+    b, c, r, _ = positions.random_positions(24, plies=100, seed=17)
+    with torch.no_grad():
+        x, alive = emulated.embed(sd, b, c, r)
+    want = co.forward(b.numpy(), c.numpy(), r.numpy(), taps=True)["resid"][:, -1]
+    got = bare(x.cuda(), alive.cuda())
+    assert got.shape == (24, 32, 256) and _bits_equal(got, want)
+    same = model.forward(x.cuda(), alive.to(torch.int8).cuda())
+    assert torch.equal(same, got)
+    half = bare(x.half().cuda(), alive.cuda())
+    assert half.dtype is torch.float16
+    # dead tokens are inert as keys: garbage in their rows changes no live row
+    x2 = x.clone()
+    x2[~alive] = 7.5
+    got2 = bare(x2.cuda(), alive.cuda())
+    assert torch.equal(got2[alive.cuda()], got[alive.cuda()])
+
+
 def test_full_batch_properties_at_4096(nets):
     # the metric's batch size: spot-check against the C checker, and size-independent properties
     net, sd, model, co = nets["seed0"]
