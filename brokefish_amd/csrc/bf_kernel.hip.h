@@ -156,7 +156,7 @@ __device__ __forceinline__ v16i mfma8(const v4i (&w)[8], const v4i (&act)[8]) {
 
 // four quotients v / sa (correctly rounded) -> round to nearest even -> low bytes packed
 __device__ __forceinline__ unsigned quant4(float v0, float v1, float v2, float v3, float sa, float inv) {
-    unsigned w = 0;
+    unsigned m[4];
     const float v[4] = {v0, v1, v2, v3};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -165,10 +165,12 @@ __device__ __forceinline__ unsigned quant4(float v0, float v1, float v2, float v
         const float rem = __builtin_fmaf(-q0, sa, v[i]);
         const float qf = __builtin_fmaf(rem, inv, q0);
         // adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low bits
-        const unsigned m = (unsigned)__float_as_int(qf + 12582912.0f);
-        w |= (m & 0xffu) << (8 * i);
+        m[i] = (unsigned)__float_as_int(qf + 12582912.0f);
     }
-    return w;
+    // gather the four low bytes with byte permutes (selector 0-3: second operand, 4-7: first, 0x0c: zero)
+    const unsigned lo = __builtin_amdgcn_perm(m[1], m[0], 0x0c0c0400u);
+    const unsigned hi = __builtin_amdgcn_perm(m[3], m[2], 0x04000c0cu);
+    return lo | hi;
 }
 
 // signed int8 quantiser of one token row spread over two lanes; y is [tiles][16]
@@ -450,6 +452,18 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                     for (int i = 0; i < 4; i++)
                         x[n][4 * j + i] = x[n][4 * j + i] + (((float)acc[4 * j + i] * so) * sw + bcur[j][i]);
                 pin16(x[n]);
+                // This tile of the residual stream is final until the FFN's last epilogue:
+                // copy it to the workspace now (one coalesced 1 KiB store per register quad),
+                // tile by tile, so the copies do not arrive at the memory system as one burst.
+                // The registers stay live through LayerNorm 2 and are released after it.
+                {
+                    float* xp = a.xpark + (size_t)board_raw * (T * D) + lane * 4;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const v4f v = {x[n][4 * j], x[n][4 * j + 1], x[n][4 * j + 2], x[n][4 * j + 3]};
+                        *reinterpret_cast<v4f*>(xp + (n * 4 + j) * 256) = v;
+                    }
+                }
                 if (TAPS && a.taps.acc_out && valid)
 #pragma unroll
                     for (int r = 0; r < 16; r++)
@@ -465,19 +479,6 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
             float y[NT][16];
             layernorm(x, lp + O_LN2G, lp + O_LN2B, a.eps, g, y);
             quant_s8<NT>(y, g, xq, sa);
-        }
-        // The residual stream is not needed again until the second FFN matmul's epilogue:
-        // park it in the workspace (one coalesced 1 KiB store per register quad) so that
-        // the hidden activations have the register file to themselves.
-        {
-            float* xp = a.xpark + (size_t)board_raw * (T * D) + lane * 4;
-#pragma unroll
-            for (int n = 0; n < NT; n++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v4f v = {x[n][4 * j], x[n][4 * j + 1], x[n][4 * j + 2], x[n][4 * j + 3]};
-                    *reinterpret_cast<v4f*>(xp + (n * 4 + j) * 256) = v;
-                }
         }
         BF_PHASE(PH_LN2);
         if (TAPS && a.taps.qa_ff1 && valid) {
@@ -542,17 +543,6 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         }
         BF_PHASE(PH_FF1);
         {
-            const float* xp = a.xpark + (size_t)board_raw * (T * D) + lane * 4;
-#pragma unroll
-            for (int n = 0; n < NT; n++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v4f v = *reinterpret_cast<const v4f*>(xp + (n * 4 + j) * 256);
-#pragma unroll
-                    for (int i = 0; i < 4; i++) x[n][4 * j + i] = v[i];
-                }
-        }
-        {
             v16i acc2[2];
             acc2[0] = BF_MM(false, 4 * NT + FT, hq[0]);
             double o64[16];
@@ -566,7 +556,17 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                 v4i wnxt[4];
                 if (idx + 1 < NT * KCF)
                     load_tile16i(lp + O_WSUM + ((idx + 1) % KCF) * D + 32 * ((idx + 1) / KCF), g, wnxt);
-                if (c == 0) load_tile16(lp + O_BFF2 + 32 * n, g, bout);   // used three blocks later
+                if (c == 0) {
+                    load_tile16(lp + O_BFF2 + 32 * n, g, bout);   // used three blocks later
+                    // bring this tile of the parked residual stream back, three blocks ahead
+                    const float* xp = a.xpark + (size_t)board_raw * (T * D) + lane * 4;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const v4f v = *reinterpret_cast<const v4f*>(xp + (n * 4 + j) * 256);
+#pragma unroll
+                        for (int i = 0; i < 4; i++) x[n][4 * j + i] = v[i];
+                    }
+                }
                 const v16i acc = acc2[idx & 1];
                 const double sc = (double)sh[c];
 #pragma unroll
