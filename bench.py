@@ -23,6 +23,9 @@ if ROOT not in sys.path:
 
 OPS_PER_EVAL = 402_653_184            # 2 * 32 tokens * 8 layers * 12 * 256^2 int8 ops in the weight GEMMs
 PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s
+# HBM bytes per launch of the default workload (batch 4096), from the FETCH_SIZE / WRITE_SIZE
+# counter runs summarised in profiles/eval_kernel_int8_batch4096.md (calibrated on a 1 GiB copy).
+MEASURED_TRAFFIC_BYTES = {4096: 3.07e9}
 
 
 def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0):
@@ -108,7 +111,8 @@ def main() -> int:
                                "seeded random playouts 0-120 plies, legal-move mask ANDed in-kernel, "
                                "fp16 logits out, seed-0 random-init weights"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
-                     "frac": achieved / (PEAK_INT8_OPS / 1e12), "traffic": None,
+                     "frac": achieved / (PEAK_INT8_OPS / 1e12),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.batch),
                      "kernel_ms": kern_ms, "ops_per_launch": OPS_PER_EVAL * a.batch},
     }
     if a.sweep:
