@@ -19,7 +19,8 @@ INCLUDE = os.path.join(ROOT, "include")
 HIP_LIB = os.path.join(HERE, "libbrokefish_hip.so")
 CHESSGEN_LIB = os.path.join(HERE, "libbf_chessgen.so")
 
-HIP_SOURCES = ["bf_host.hip", "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip"]
+HIP_SOURCES = ["bf_host.hip", "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip",
+               "bf_variant_prod_fp8.hip", "bf_variant_taps_fp8.hip"]
 # -ffp-contract=off: the kernel's fp32 arithmetic is specified operation by operation
 # (fused multiply-adds are written explicitly), so the compiler must not fuse on its own.
 # The packed-fp32 feature is disabled so no v_pk_*_f32 instructions are generated.

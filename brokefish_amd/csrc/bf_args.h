@@ -56,7 +56,7 @@ static_assert(LAYER_BLOCKS % 8 == 0, "ring slot of a block must not depend on th
 constexpr int O_LN1G = 0, O_LN1B = D, O_BQKV = 2 * D, O_BOUT = 5 * D, O_LN2G = 6 * D,
               O_LN2B = 7 * D, O_BFF1 = 8 * D, O_BFF2 = 8 * D + F, O_WSUM = 9 * D + F,
               O_SW = 9 * D + F + KCF * D;
-constexpr int N_SW = 3 * D / 128 + D / 128 + F / 128 + D / 128;
+constexpr int N_SW = 3 * D / 128 + D / 128 + F / 128 + (D / 128) * KCF;   // ffn2: one per (128-row block, k-chunk)
 constexpr int LAYER_FLOATS = O_SW + ((N_SW + 3) / 4) * 4;
 // a layer's parameters are padded to a whole number of 4 KiB copies (one per workgroup pass)
 constexpr int PARAM_BYTES = ((LAYER_FLOATS * 4 + WAVES * FRAG - 1) / (WAVES * FRAG)) * (WAVES * FRAG);
@@ -96,5 +96,7 @@ struct KArgs {
 hipError_t launch_prod(const KArgs& k, int grid, hipStream_t stream);
 hipError_t launch_taps(const KArgs& k, int grid, hipStream_t stream);
 hipError_t launch_prof(const KArgs& k, int grid, hipStream_t stream);
+hipError_t launch_prod_fp8(const KArgs& k, int grid, hipStream_t stream);
+hipError_t launch_taps_fp8(const KArgs& k, int grid, hipStream_t stream);
 
 }  // namespace bf

@@ -46,6 +46,8 @@ extern "C" void bf_int8_q_max(double* s8, double* u8) {
     if (u8) *u8 = 255.0;
 }
 
+extern "C" double bf_fp8_q_max(void) { return 8.0; }
+
 extern "C" const char* bf_last_error(void) { return g_err; }
 
 static int check_args(const bf_eval_args* a, bf::KArgs* k) {
@@ -63,6 +65,8 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k) {
     if (((uintptr_t)a->policy & 15) || ((uintptr_t)a->promo & 7) || ((uintptr_t)a->boards & 1))
         return fail(BF_ERR_ARGUMENT, "policy must be 16-byte and promo 8-byte aligned");
     if (a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
+    if (a->quant != BF_QUANT_INT8 && a->quant != BF_QUANT_E4M3)
+        return fail(BF_ERR_ARGUMENT, "quant must be BF_QUANT_INT8 or BF_QUANT_E4M3");
     if (!a->workspace || ((uintptr_t)a->workspace & 15) || a->workspace_bytes < bf_workspace_bytes(&a->shape, a->n))
         return fail(BF_ERR_ARGUMENT, "workspace must be 16-byte aligned and hold bf_workspace_bytes(shape, n) bytes");
     memset(k, 0, sizeof(*k));
@@ -88,9 +92,13 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k) {
 
 static int launch(const bf_eval_args* a, const bf::KArgs& k, hipStream_t stream) {
     const int grid = (k.n + bf::WAVES - 1) / bf::WAVES;
-    const hipError_t e = k.profile ? bf::launch_prof(k, grid, stream)
-                       : a->taps   ? bf::launch_taps(k, grid, stream)
-                                   : bf::launch_prod(k, grid, stream);
+    hipError_t e;
+    if (a->quant == BF_QUANT_E4M3)
+        e = a->taps ? bf::launch_taps_fp8(k, grid, stream) : bf::launch_prod_fp8(k, grid, stream);
+    else
+        e = k.profile ? bf::launch_prof(k, grid, stream)
+          : a->taps   ? bf::launch_taps(k, grid, stream)
+                      : bf::launch_prod(k, grid, stream);
     if (e != hipSuccess) {
         snprintf(g_err, sizeof(g_err), "kernel launch failed: %s", hipGetErrorString(e));
         return BF_ERR_LAUNCH;
@@ -110,6 +118,7 @@ extern "C" int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_
     const int rc = check_args(args, &k);
     if (rc) return rc;
     if (args->taps) return fail(BF_ERR_ARGUMENT, "the phase profile runs without taps");
+    if (args->quant != BF_QUANT_INT8) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the int8 format only");
     if (!cycles) return fail(BF_ERR_ARGUMENT, "cycles must not be NULL");
     k.profile = reinterpret_cast<unsigned long long*>(cycles);
     return launch(args, k, (hipStream_t)stream);

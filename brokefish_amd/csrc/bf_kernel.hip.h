@@ -5,8 +5,11 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "bf_args.h"
 
+typedef long v2l __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -141,40 +144,79 @@ __device__ __forceinline__ void load_frags(int blk, v4i (&fr)[8], Stream& st, in
     for (int s = 0; s < 8; s++) fr[s] = *reinterpret_cast<const v4i*>(&ring[off + s * FRAG + lane * 16]);
 }
 
-// acc[out_channel r][token] (weights as A) or acc[token r][out_channel] (SWAP, weights as B)
-template <bool SWAP>
-__device__ __forceinline__ v16i mfma8(const v4i (&w)[8], const v4i (&act)[8]) {
-    v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+// acc[out_channel r][token] (weights as A) or acc[token r][out_channel] (SWAP, weights as B).
+// int8: eight v_mfma_i32_32x32x32_i8; e4m3: each 16-byte fragment is two k-steps of
+// v_mfma_f32_32x32x16_fp8_fp8 (the same lane/byte pairing, so the packing is shared).
+template <bool FP8> struct Acc { typedef v16i type; };
+template <> struct Acc<true> { typedef v16f type; };
+
+template <bool SWAP, bool FP8>
+__device__ __forceinline__ typename Acc<FP8>::type mfma8(const v4i (&w)[8], const v4i (&act)[8]) {
+    if constexpr (FP8) {
+        v16f acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int s = 0; s < 8; s++)
-        acc = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act[s], w[s], acc, 0, 0, 0)
-                   : __builtin_amdgcn_mfma_i32_32x32x32_i8(w[s], act[s], acc, 0, 0, 0);
-    return acc;
+        for (int s = 0; s < 8; s++) {
+            const v2l wl = __builtin_bit_cast(v2l, w[s]);
+            const v2l al = __builtin_bit_cast(v2l, act[s]);
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++)
+                acc = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[hlf], wl[hlf], acc, 0, 0, 0)
+                           : __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(wl[hlf], al[hlf], acc, 0, 0, 0);
+        }
+        return acc;
+    } else {
+        v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+            acc = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act[s], w[s], acc, 0, 0, 0)
+                       : __builtin_amdgcn_mfma_i32_32x32x32_i8(w[s], act[s], acc, 0, 0, 0);
+        return acc;
+    }
 }
+
+// accumulator element as fp32 (exact for the int32 accumulators: they stay below 2^24)
+__device__ __forceinline__ float accf(const v16i& a, int i) { return (float)a[i]; }
+__device__ __forceinline__ float accf(const v16f& a, int i) { return a[i]; }
+__device__ __forceinline__ int accbits(const v16i& a, int i) { return a[i]; }
+__device__ __forceinline__ int accbits(const v16f& a, int i) { return __float_as_int(a[i]); }
 
 // ---- row operations -------------------------------------------------------------------
 
-// four quotients v / sa (correctly rounded) -> round to nearest even -> low bytes packed
+// four quotients v / sa (correctly rounded) -> one packed dword.
+// int8: round to nearest even, low bytes gathered.  e4m3: clamp to the format's range and
+// convert with the hardware's round-to-nearest-even OCP e4m3 conversion.
+template <bool FP8>
 __device__ __forceinline__ unsigned quant4(float v0, float v1, float v2, float v3, float sa, float inv) {
-    unsigned m[4];
+    float qf[4];
     const float v[4] = {v0, v1, v2, v3};
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         // correctly rounded v / sa from the reciprocal and two fused corrections
         const float q0 = v[i] * inv;
         const float rem = __builtin_fmaf(-q0, sa, v[i]);
-        const float qf = __builtin_fmaf(rem, inv, q0);
-        // adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low bits
-        m[i] = (unsigned)__float_as_int(qf + 12582912.0f);
+        qf[i] = __builtin_fmaf(rem, inv, q0);
     }
-    // gather the four low bytes with byte permutes (selector 0-3: second operand, 4-7: first, 0x0c: zero)
-    const unsigned lo = __builtin_amdgcn_perm(m[1], m[0], 0x0c0c0400u);
-    const unsigned hi = __builtin_amdgcn_perm(m[3], m[2], 0x04000c0cu);
-    return lo | hi;
+    if constexpr (FP8) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) qf[i] = __builtin_fminf(__builtin_fmaxf(qf[i], -448.0f), 448.0f);
+        int w = __builtin_amdgcn_cvt_pk_fp8_f32(qf[0], qf[1], 0, false);
+        w = __builtin_amdgcn_cvt_pk_fp8_f32(qf[2], qf[3], w, true);
+        return (unsigned)w;
+    } else {
+        unsigned m[4];
+        // adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low bits
+#pragma unroll
+        for (int i = 0; i < 4; i++) m[i] = (unsigned)__float_as_int(qf[i] + 12582912.0f);
+        // gather the four low bytes with byte permutes (selector 0-3: second operand, 4-7: first, 0x0c: zero)
+        const unsigned lo = __builtin_amdgcn_perm(m[1], m[0], 0x0c0c0400u);
+        const unsigned hi = __builtin_amdgcn_perm(m[3], m[2], 0x04000c0cu);
+        return lo | hi;
+    }
 }
 
-// signed int8 quantiser of one token row spread over two lanes; y is [tiles][16]
-template <int NTILES>
+// signed quantiser (int8: amax -> 127, e4m3: amax -> 8) of one token row spread over two
+// lanes; y is [tiles][16]
+template <int NTILES, bool FP8>
 __device__ __forceinline__ void quant_s8(const float (&y)[NTILES][16], int g, v4i (&q)[NTILES], float& sa) {
     float am = 0.0f;
 #pragma unroll
@@ -182,13 +224,13 @@ __device__ __forceinline__ void quant_s8(const float (&y)[NTILES][16], int g, v4
 #pragma unroll
         for (int r = 0; r < 16; r++) am = __builtin_fmaxf(am, __builtin_fabsf(y[n][r]));
     am = __builtin_fmaxf(am, partner(am, g));
-    sa = am > 0.0f ? am / 127.0f : 1.0f;
+    sa = am > 0.0f ? am / (FP8 ? 8.0f : 127.0f) : 1.0f;
     const float inv = 1.0f / sa;
 #pragma unroll
     for (int n = 0; n < NTILES; n++)
 #pragma unroll
         for (int j = 0; j < 4; j++)
-            q[n][j] = (int)quant4(y[n][4 * j], y[n][4 * j + 1], y[n][4 * j + 2], y[n][4 * j + 3], sa, inv);
+            q[n][j] = (int)quant4<FP8>(y[n][4 * j], y[n][4 * j + 1], y[n][4 * j + 2], y[n][4 * j + 3], sa, inv);
 }
 
 // LayerNorm of the residual rows, affine applied, in the fixed lane order; gamma/beta in LDS or global
@@ -226,8 +268,9 @@ __device__ __forceinline__ void layernorm(const float (&x)[NT][16], const float*
 
 // ---- the kernel ------------------------------------------------------------------------
 
-template <bool TAPS, bool PROF>
+template <bool TAPS, bool PROF, bool FP8>
 __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
+    typedef typename Acc<FP8>::type acc_t;
     unsigned long long ph[N_PHASES];
     unsigned long long t_mark = 0, t_begin = 0;
     if (PROF) {
@@ -330,8 +373,8 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         const bool more = l + 1 < a.l1;
         // multiply by the block in `fr`, then fetch the fragments of the block after it
 #define BF_MM(SWAP, blk, act)                                                   \
-    ([&]() -> v16i {                                                            \
-        const v16i r_ = mfma8<SWAP>(fr, act);                                   \
+    ([&]() -> acc_t {                                                           \
+        const acc_t r_ = mfma8<SWAP, FP8>(fr, act);                             \
         if ((blk) + 1 < LAYER_BLOCKS || more) load_frags<PROF>((blk) + 1, fr, st, wave, lane); \
         return r_;                                                              \
     }())
@@ -341,7 +384,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         {
             float y[NT][16];
             layernorm(x, lp + O_LN1G, lp + O_LN1B, a.eps, g, y);
-            quant_s8<NT>(y, g, xq, sa);
+            quant_s8<NT, FP8>(y, g, xq, sa);
         }
         if (TAPS && a.taps.qa_qkv && valid) {
 #pragma unroll
@@ -356,41 +399,40 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; r++) sa_tok[r] = __shfl(sa, ch(r, g));
 
-        // ---- attention, one head at a time ------------------------------------------------
+        // ---- attention, one head at a time, software-pipelined ---------------------------------
+        // The three weight GEMMs of head h+1 are issued right after the score MFMAs of head h,
+        // so the matrix pipe works through them while the vector ALU does head h's softmax, and
+        // head h's PV MFMAs run under head h+1's epilogue.
         float o[NH][16];
+        acc_t accq = BF_MM(false, 0, xq);
+        acc_t acck = BF_MM(false, 1, xq);
+        acc_t accv = BF_MM(true, 2, xq);   // V transposed: lane = channel, registers = tokens
 #pragma unroll
         for (int h = 0; h < NH; h++) {
-            // parameters of this head's three tiles, fetched ahead of the matrix products
-            const float swq = lp[O_SW + SW_QKV + (32 * h) / 128];
-            const float swk = lp[O_SW + SW_QKV + (D + 32 * h) / 128];
-            const float swv = lp[O_SW + SW_QKV + (2 * D + 32 * h) / 128];
-            const float bv = lp[O_BQKV + 2 * D + 32 * h + t];
-            v4f bq[4], bk[4];
-            load_tile16(lp + O_BQKV + 32 * h, g, bq);
-            load_tile16(lp + O_BQKV + D + 32 * h, g, bk);
-            const v16i accq = BF_MM(false, 3 * h + 0, xq);
-            const v16i acck = BF_MM(false, 3 * h + 1, xq);
-            const v16i accv = BF_MM(true, 3 * h + 2, xq);   // V transposed: lane = channel, registers = tokens
-            // The next layer's parameters can be fetched once every wave is inside this layer
-            // (after the last layer the same layer is fetched again, into the idle buffer).
-            if (h == 1) issue_params(a.fparams, more ? l + 1 : l, (li + 1) & 1, wave, lane);
             float qf[16], kf[16], vf[16];
             {
+                const float swq = lp[O_SW + SW_QKV + (32 * h) / 128];
+                const float swk = lp[O_SW + SW_QKV + (D + 32 * h) / 128];
+                const float swv = lp[O_SW + SW_QKV + (2 * D + 32 * h) / 128];
+                const float bv = lp[O_BQKV + 2 * D + 32 * h + t];
+                v4f bq[4], bk[4];
+                load_tile16(lp + O_BQKV + 32 * h, g, bq);
+                load_tile16(lp + O_BQKV + D + 32 * h, g, bk);
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        qf[4 * j + i] = ((float)accq[4 * j + i] * sa) * swq + bq[j][i];
-                        kf[4 * j + i] = ((float)acck[4 * j + i] * sa) * swk + bk[j][i];
+                        qf[4 * j + i] = (accf(accq, 4 * j + i) * sa) * swq + bq[j][i];
+                        kf[4 * j + i] = (accf(acck, 4 * j + i) * sa) * swk + bk[j][i];
                     }
 #pragma unroll
-                for (int r = 0; r < 16; r++) vf[r] = ((float)accv[r] * sa_tok[r]) * swv + bv;
+                for (int r = 0; r < 16; r++) vf[r] = (accf(accv, r) * sa_tok[r]) * swv + bv;
                 if (TAPS && a.taps.acc_qkv && valid)
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        a.taps.acc_qkv[(bl * T + t) * 3 * D + 32 * h + ch(r, g)] = accq[r];
-                        a.taps.acc_qkv[(bl * T + t) * 3 * D + D + 32 * h + ch(r, g)] = acck[r];
-                        a.taps.acc_qkv[(bl * T + ch(r, g)) * 3 * D + 2 * D + 32 * h + t] = accv[r];
+                        a.taps.acc_qkv[(bl * T + t) * 3 * D + 32 * h + ch(r, g)] = accbits(accq, r);
+                        a.taps.acc_qkv[(bl * T + t) * 3 * D + D + 32 * h + ch(r, g)] = accbits(acck, r);
+                        a.taps.acc_qkv[(bl * T + ch(r, g)) * 3 * D + 2 * D + 32 * h + t] = accbits(accv, r);
                     }
             }
             BF_PHASE(PH_QKV);
@@ -398,6 +440,14 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
             v16f sc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
             for (int r = 0; r < 16; r++) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[r], qf[r], sc, 0, 0, 0);
+            if (h + 1 < NH) {
+                accq = BF_MM(false, 3 * (h + 1) + 0, xq);
+                acck = BF_MM(false, 3 * (h + 1) + 1, xq);
+                accv = BF_MM(true, 3 * (h + 1) + 2, xq);
+            }
+            // The next layer's parameters can be fetched once every wave is inside this layer
+            // (after the last layer the same layer is fetched again, into the idle buffer).
+            if (h == 1) issue_params(a.fparams, more ? l + 1 : l, (li + 1) & 1, wave, lane);
             float p[16];
             float mx = -__builtin_inff();
 #pragma unroll
@@ -427,7 +477,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         {
             v4i oq[NT];
             float so;
-            quant_s8<NT>(o, g, oq, so);
+            quant_s8<NT, FP8>(o, g, oq, so);
             if (TAPS && a.taps.qa_out && valid) {
 #pragma unroll
                 for (int n = 0; n < NT; n++)
@@ -435,7 +485,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                     for (int j = 0; j < 4; j++)
                         *reinterpret_cast<int*>(a.taps.qa_out + (bl * T + t) * D + 32 * n + 8 * j + 4 * g) = oq[n][j];
             }
-            v16i acc2[2];
+            acc_t acc2[2];
             acc2[0] = BF_MM(false, 3 * NT, oq);
             v4f bcur[4];
             load_tile16(lp + O_BOUT, g, bcur);
@@ -444,13 +494,13 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                 if (n + 1 < NT) acc2[(n + 1) & 1] = BF_MM(false, 3 * NT + n + 1, oq);
                 v4f bnxt[4];   // parameters are fetched one tile ahead of their use
                 if (n + 1 < NT) load_tile16(lp + O_BOUT + 32 * (n + 1), g, bnxt);
-                const v16i acc = acc2[n & 1];
+                const acc_t acc = acc2[n & 1];
                 const float sw = lp[O_SW + SW_OUT + (32 * n) / 128];
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int i = 0; i < 4; i++)
-                        x[n][4 * j + i] = x[n][4 * j + i] + (((float)acc[4 * j + i] * so) * sw + bcur[j][i]);
+                        x[n][4 * j + i] = x[n][4 * j + i] + ((accf(acc, 4 * j + i) * so) * sw + bcur[j][i]);
                 pin16(x[n]);
                 // This tile of the residual stream is final until the FFN's last epilogue:
                 // copy it to the workspace now (one coalesced 1 KiB store per register quad),
@@ -467,7 +517,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                 if (TAPS && a.taps.acc_out && valid)
 #pragma unroll
                     for (int r = 0; r < 16; r++)
-                        a.taps.acc_out[(bl * T + t) * D + 32 * n + ch(r, g)] = acc[r];
+                        a.taps.acc_out[(bl * T + t) * D + 32 * n + ch(r, g)] = accbits(acc, r);
 #pragma unroll
                 for (int j = 0; j < 4; j++) bcur[j] = bnxt[j];
             }
@@ -478,7 +528,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         {
             float y[NT][16];
             layernorm(x, lp + O_LN2G, lp + O_LN2B, a.eps, g, y);
-            quant_s8<NT>(y, g, xq, sa);
+            quant_s8<NT, FP8>(y, g, xq, sa);
         }
         BF_PHASE(PH_LN2);
         if (TAPS && a.taps.qa_ff1 && valid) {
@@ -491,7 +541,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         v4i hq[KCF][8];
         float sh[KCF];
         {
-            v16i acc2[2];
+            acc_t acc2[2];
             acc2[0] = BF_MM(false, 4 * NT, xq);
             float hf[8][16];
             float am = 0.0f;
@@ -503,13 +553,13 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                 if (tile + 1 < FT) acc2[(tile + 1) & 1] = BF_MM(false, 4 * NT + tile + 1, xq);
                 v4f bnxt[4];
                 if (tile + 1 < FT) load_tile16(lp + O_BFF1 + 32 * (tile + 1), g, bnxt);
-                const v16i acc = acc2[tile & 1];
+                const acc_t acc = acc2[tile & 1];
                 const float sw = lp[O_SW + SW_FF1 + (32 * tile) / 128];
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const float v = __builtin_fmaxf(((float)acc[4 * j + i] * sa) * sw + bcur[j][i], 0.0f);
+                        const float v = __builtin_fmaxf((accf(acc, 4 * j + i) * sa) * sw + bcur[j][i], 0.0f);
                         hf[s][4 * j + i] = v;
                         am = __builtin_fmaxf(am, v);
                     }
@@ -519,23 +569,24 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                 if (TAPS && a.taps.acc_ff1 && valid)
 #pragma unroll
                     for (int r = 0; r < 16; r++)
-                        a.taps.acc_ff1[(bl * T + t) * F + 32 * tile + ch(r, g)] = acc[r];
+                        a.taps.acc_ff1[(bl * T + t) * F + 32 * tile + ch(r, g)] = accbits(acc, r);
                 if (s == 7) {
-                    // unsigned quantiser over this 256-wide chunk; bytes stored as q - 128 for
-                    // the signed MFMA, the offset is added back through wsum
+                    // int8: unsigned quantiser over this 256-wide chunk; bytes stored as q - 128
+                    // for the signed MFMA, the offset is added back through wsum.
+                    // e4m3: the ordinary signed quantiser (the values are non-negative).
                     am = __builtin_fmaxf(am, partner(am, g));
-                    const float s8 = am > 0.0f ? am / 255.0f : 1.0f;
+                    const float s8 = am > 0.0f ? am / (FP8 ? 8.0f : 255.0f) : 1.0f;
                     const float inv = 1.0f / s8;
                     sh[c] = s8;
 #pragma unroll
                     for (int s2 = 0; s2 < 8; s2++)
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
-                            const unsigned w = quant4(hf[s2][4 * j], hf[s2][4 * j + 1], hf[s2][4 * j + 2],
-                                                      hf[s2][4 * j + 3], s8, inv);
+                            const unsigned w = quant4<FP8>(hf[s2][4 * j], hf[s2][4 * j + 1], hf[s2][4 * j + 2],
+                                                           hf[s2][4 * j + 3], s8, inv);
                             if (TAPS && a.taps.qa_ff2 && valid)
                                 *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 256 * c + 32 * s2 + 8 * j + 4 * g) = w;
-                            hq[c][s2][j] = (int)(w ^ 0x80808080u);
+                            hq[c][s2][j] = (int)(FP8 ? w : (w ^ 0x80808080u));
                         }
                     am = 0.0f;
                 }
@@ -543,18 +594,19 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
         }
         BF_PHASE(PH_FF1);
         {
-            v16i acc2[2];
+            acc_t acc2[2];
             acc2[0] = BF_MM(false, 4 * NT + FT, hq[0]);
-            double o64[16];
+            double o64[16];   // int8: float64 sum over the k-chunks, as the reference's emulation
+            float o32[16];    // e4m3: fp32 sum over the k-tiles
             v4i wcur[4];
-            load_tile16i(lp + O_WSUM, g, wcur);
+            if (!FP8) load_tile16i(lp + O_WSUM, g, wcur);
             v4f bout[4];
 #pragma unroll
             for (int idx = 0; idx < NT * KCF; idx++) {
                 const int n = idx / KCF, c = idx % KCF;
                 if (idx + 1 < NT * KCF) acc2[(idx + 1) & 1] = BF_MM(false, 4 * NT + FT + idx + 1, hq[(idx + 1) % KCF]);
                 v4i wnxt[4];
-                if (idx + 1 < NT * KCF)
+                if (!FP8 && idx + 1 < NT * KCF)
                     load_tile16i(lp + O_WSUM + ((idx + 1) % KCF) * D + 32 * ((idx + 1) / KCF), g, wnxt);
                 if (c == 0) {
                     load_tile16(lp + O_BFF2 + 32 * n, g, bout);   // used three blocks later
@@ -567,33 +619,52 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                         for (int i = 0; i < 4; i++) x[n][4 * j + i] = v[i];
                     }
                 }
-                const v16i acc = acc2[idx & 1];
-                const double sc = (double)sh[c];
+                const acc_t acc = acc2[idx & 1];
+                // weight scale of this (128-row block, k-chunk); int8 packs the same value for every chunk
+                const float sw = lp[O_SW + SW_FF2 + ((32 * n) / 128) * KCF + c];
+                if constexpr (FP8) {
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int full = acc[4 * j + i] + wcur[j][i];
-                        // exact product, one rounding in the add: same as out += acc * sa in fp64
-                        o64[4 * j + i] = c == 0 ? (double)full * sc
-                                                : __builtin_fma((double)full, sc, o64[4 * j + i]);
+                    for (int i = 0; i < 16; i++) {
+                        const float part = (accf(acc, i) * sh[c]) * sw;
+                        o32[i] = c == 0 ? part : o32[i] + part;
                         if (TAPS && a.taps.acc_ff2 && valid)
-                            a.taps.acc_ff2[((bl * KCF + c) * T + t) * D + 32 * n + 8 * j + 4 * g + i] = full;
+                            a.taps.acc_ff2[((bl * KCF + c) * T + t) * D + 32 * n + ch(i, g)] = accbits(acc, i);
                     }
-                if (c == KCF - 1) {
-                    const float sw = lp[O_SW + SW_FF2 + (32 * n) / 128];
+                } else {
+                    const double sc = (double)sh[c];
 #pragma unroll
                     for (int j = 0; j < 4; j++)
 #pragma unroll
-                        for (int i = 0; i < 4; i++)
-                            x[n][4 * j + i] = x[n][4 * j + i] + ((float)o64[4 * j + i] * sw + bout[j][i]);
+                        for (int i = 0; i < 4; i++) {
+                            const int full = accbits(acc, 4 * j + i) + wcur[j][i];
+                            // exact product, one rounding in the add: same as out += acc * sa in fp64
+                            o64[4 * j + i] = c == 0 ? (double)full * sc
+                                                    : __builtin_fma((double)full, sc, o64[4 * j + i]);
+                            if (TAPS && a.taps.acc_ff2 && valid)
+                                a.taps.acc_ff2[((bl * KCF + c) * T + t) * D + 32 * n + 8 * j + 4 * g + i] = full;
+                        }
+                }
+                if (c == KCF - 1) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            float upd;
+                            if constexpr (FP8) upd = o32[4 * j + i] + bout[j][i];
+                            else upd = (float)o64[4 * j + i] * sw + bout[j][i];
+                            x[n][4 * j + i] = x[n][4 * j + i] + upd;
+                        }
                     pin16(x[n]);
+                } else if constexpr (FP8) {
+                    pin16(o32);
                 } else {
 #pragma unroll
                     for (int i = 0; i < 16; i++) pin(o64[i]);
                 }
+                if (!FP8) {
 #pragma unroll
-                for (int j = 0; j < 4; j++) wcur[j] = wnxt[j];
+                    for (int j = 0; j < 4; j++) wcur[j] = wnxt[j];
+                }
             }
         }
 #undef BF_MM
@@ -713,17 +784,17 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
 }
 
 
-template <bool TAPS, bool PROF>
+template <bool TAPS, bool PROF, bool FP8>
 hipError_t launch_variant(const KArgs& k, int grid, hipStream_t stream) {
     // more than 64 KiB of dynamic LDS has to be requested once per kernel (per thread: cheap)
     static thread_local bool lds_set = false;
     if (!lds_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&eval_kernel<TAPS, PROF>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&eval_kernel<TAPS, PROF, FP8>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (e != hipSuccess) return e;
         lds_set = true;
     }
-    hipLaunchKernelGGL((eval_kernel<TAPS, PROF>), dim3(grid), dim3(THREADS), LDS_BYTES, stream, k);
+    hipLaunchKernelGGL((eval_kernel<TAPS, PROF, FP8>), dim3(grid), dim3(THREADS), LDS_BYTES, stream, k);
     return hipGetLastError();
 }
 

@@ -2,5 +2,5 @@
 #include "bf_kernel.hip.h"
 
 namespace bf {
-hipError_t launch_prod(const KArgs& k, int grid, hipStream_t stream) { return launch_variant<false, false>(k, grid, stream); }
+hipError_t launch_prod(const KArgs& k, int grid, hipStream_t stream) { return launch_variant<false, false, false>(k, grid, stream); }
 }  // namespace bf

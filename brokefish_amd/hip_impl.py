@@ -32,6 +32,9 @@ from . import _build
 T, N_POLICY, N_PROMO = 32, 64, 4
 BLOCK_N = 128            # weight-scale block, brokefish/nn/quant.py:82
 Q_MAX_S8, Q_MAX_U8 = 127.0, 255.0   # brokefish/nn/quant.py:237-241
+ROW_K = 256              # k-depth one e4m3 activation scale covers, brokefish/nn/quant.py:92
+Q_MAX_E4M3 = 8.0         # what a row's / block's maximum maps to in e4m3, brokefish/nn/quant.py:105
+E4M3_MAX = 448.0         # largest finite e4m3 value, brokefish/nn/quant.py:73
 
 
 class _Shape(C.Structure):
@@ -53,7 +56,7 @@ class _Args(C.Structure):
                 ("mask", C.c_void_p), ("n", C.c_int64), ("shape", _Shape),
                 ("wstream", C.c_void_p), ("fparams", C.c_void_p),
                 ("policy", C.c_void_p), ("promo", C.c_void_p), ("value", C.c_void_p),
-                ("best_move", C.c_void_p), ("out_fp32", C.c_int32),
+                ("best_move", C.c_void_p), ("out_fp32", C.c_int32), ("quant", C.c_int32),
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("taps", C.POINTER(_Taps))]
 
 
@@ -89,6 +92,7 @@ def load_library():
         L.bf_profile_phase_name.restype = C.c_char_p
         L.bf_profile_phase_name.argtypes = [C.c_int]
         L.bf_int8_q_max.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_double)]
+        L.bf_fp8_q_max.restype = C.c_double
         _lib = L
     return _lib
 
@@ -98,6 +102,11 @@ def int8_q_max():
     a, b = C.c_double(), C.c_double()
     load_library().bf_int8_q_max(C.byref(a), C.byref(b))
     return a.value, b.value
+
+
+def fp8_q_max() -> float:
+    """The e4m3 quantisation maximum compiled into the library."""
+    return float(load_library().bf_fp8_q_max())
 
 
 # --------------------------------------------------------------------------- #
@@ -115,6 +124,20 @@ def quantise_weights_int8(w: torch.Tensor):
     scale = torch.where(amax > 0, amax / Q_MAX_S8, torch.ones_like(amax))
     q = torch.round(blocks / scale).clamp(-Q_MAX_S8, Q_MAX_S8).to(torch.int8)
     return q.reshape(n, k).numpy(), scale.reshape(-1).numpy().astype(np.float32)
+
+
+def quantise_weights_e4m3(w: torch.Tensor):
+    """[N, K] fp32 -> (e4m3 bytes uint8 [N, K], fp32 scale [N // 128, K // 256]); one scale
+    per 128-row x 256-deep block whose largest magnitude lands on 8
+    (brokefish/nn/quant.py:208-224 with q_max = Q_MAX, tile_k = ROW_K)."""
+    n, k = w.shape
+    if n % BLOCK_N or k % ROW_K:
+        raise ValueError(f"weight {tuple(w.shape)} does not tile into {BLOCK_N}x{ROW_K} blocks")
+    blocks = w.detach().float().cpu().reshape(n // BLOCK_N, BLOCK_N, k // ROW_K, ROW_K)
+    amax = blocks.abs().amax(dim=(1, 3), keepdim=True)
+    scale = torch.where(amax > 0, amax / Q_MAX_E4M3, torch.ones_like(amax))
+    q = (blocks / scale).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn).reshape(n, k)
+    return q.view(torch.uint8).numpy(), scale.reshape(n // BLOCK_N, k // ROW_K).numpy().astype(np.float32)
 
 
 def _lane_tables():
@@ -147,10 +170,12 @@ def pack_head_tile(head: np.ndarray, m: int) -> np.ndarray:
 
 
 def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_value: int,
-                 layer_stride: Optional[int] = None):
+                 layer_stride: Optional[int] = None, fmt: str = "int8"):
     """state_dict -> (wstream uint8 [bytes], fparams float32 [floats]) in the layouts of
     include/brokefish_hip.h.  ``layer_stride`` is the per-layer stride of fparams in floats
-    (default: what the library reports for this shape)."""
+    (default: what the library reports for this shape); ``fmt`` is "int8" or "e4m3"."""
+    if fmt not in ("int8", "e4m3"):
+        raise ValueError(f"fmt = {fmt!r}, expected 'int8' or 'e4m3'")
     if layer_stride is None:
         shape = _Shape(d, n_layers, d // 32, f, n_value, 1e-5)
         layer_stride = int(load_library().bf_layer_stride_floats(C.byref(shape)))
@@ -161,10 +186,18 @@ def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_v
     stream, fl = [], []
     for l in range(n_layers):
         p = f"encoder.layers.{l}."
-        q_qkv, s_qkv = quantise_weights_int8(get(p + "self_attn.in_proj_weight"))
-        q_out, s_out = quantise_weights_int8(get(p + "self_attn.out_proj.weight"))
-        q_ff1, s_ff1 = quantise_weights_int8(get(p + "linear1.weight"))
-        q_ff2, s_ff2 = quantise_weights_int8(get(p + "linear2.weight"))
+        names = ("self_attn.in_proj_weight", "self_attn.out_proj.weight", "linear1.weight", "linear2.weight")
+        if fmt == "int8":
+            (q_qkv, s_qkv), (q_out, s_out), (q_ff1, s_ff1), (q_ff2, s_ff2) = \
+                [quantise_weights_int8(get(p + nm)) for nm in names]
+            # the scale table carries one ffn2 entry per (128-row block, k-chunk): the int8
+            # scheme scales over the whole reduction, so its value repeats
+            s_ff2 = np.repeat(s_ff2[:, None], kcf, axis=1)
+            wsum = (128 * q_ff2.astype(np.int32).reshape(d, kcf, 256).sum(axis=2)).T   # [kcf, d]
+        else:
+            (q_qkv, s_qkv), (q_out, s_out), (q_ff1, s_ff1), (q_ff2, s_ff2) = \
+                [quantise_weights_e4m3(get(p + nm)) for nm in names]
+            wsum = np.zeros((kcf, d), np.int32)      # no unsigned operand in this format
         for h in range(nt):
             for part in range(3):
                 stream.append(pack_int8_block(q_qkv, part * nt + h, 0))
@@ -175,8 +208,7 @@ def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_v
         for n in range(nt):
             for c in range(kcf):
                 stream.append(pack_int8_block(q_ff2, n, 256 * c))
-        wsum = (128 * q_ff2.astype(np.int32).reshape(d, kcf, 256).sum(axis=2)).T   # [kcf, d]
-        sw = np.concatenate([s_qkv, s_out, s_ff1, s_ff2]).astype(np.float32)
+        sw = np.concatenate([np.reshape(x, -1) for x in (s_qkv, s_out, s_ff1, s_ff2)]).astype(np.float32)
         sw = np.concatenate([sw, np.zeros((-len(sw)) % 4, np.float32)])
         layer = [get(p + "norm1.weight").numpy(), get(p + "norm1.bias").numpy(),
                  get(p + "self_attn.in_proj_bias").numpy(), get(p + "self_attn.out_proj.bias").numpy(),
@@ -222,11 +254,10 @@ class FusedEncoder:
             raise ValueError(f"acc_dtype must be one of {self.ACC_DTYPES}, got {acc_dtype!r}")
         if fp8 and int8:
             raise ValueError("fp8 and int8 quantise the same matmuls; pick one")
-        if fp8:
-            raise NotImplementedError("this build carries the int8 evaluator only (no e4m3 path yet)")
-        if int8 is False:
+        if int8 is False and not fp8:
             raise NotImplementedError(
-                "this build carries the int8 evaluator only; construct with int8=True (the default here)")
+                "this build carries the quantised evaluators only; construct with int8=True "
+                "(the default here) or fp8=True")
         if int8_scheme != "all":
             raise NotImplementedError(
                 "all four matmuls of every layer are int8 here, which is the reference's 'all' scheme")
@@ -258,8 +289,9 @@ class FusedEncoder:
         self.n_value = int(net.value.weight.shape[0]) if net is not None else 1
         if self.n_value not in (1, 3):
             raise ValueError(f"value head must have 1 or 3 rows, got {self.n_value}")
-        self.acc_dtype, self.fp8, self.int8 = acc_dtype, False, True
-        self.int8_scheme, self.quant = int8_scheme, 3
+        self.acc_dtype, self.fp8, self.int8 = acc_dtype, bool(fp8), not fp8
+        # `quant` keeps the reference's numbering (1: e4m3, 3: int8 on all four matmuls)
+        self.int8_scheme, self.quant = int8_scheme, (1 if fp8 else 3)
         # Boards per workgroup is an occupancy detail of this kernel (four); the flag is
         # accepted for signature compatibility and changes no number.
         self.two_boards = True if two_boards is None else bool(two_boards)
@@ -280,7 +312,8 @@ class FusedEncoder:
                                ("emb_clock", 101), ("emb_rep", 3), ("policy", 64), ("promo", 4), ("value", 1)):
                 sd[name + ".weight"] = torch.zeros(rows, d)
             sd["norm_f.weight"], sd["norm_f.bias"] = torch.ones(d), torch.zeros(d)
-        wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value)
+        wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value,
+                                        fmt="e4m3" if self.fp8 else "int8")
         if wstream.size != self._lib.bf_wstream_bytes(C.byref(self._shape)) or \
                 fparams.size != self._lib.bf_fparams_floats(C.byref(self._shape)):
             raise RuntimeError("packed blob sizes disagree with the library's layout")
@@ -291,7 +324,8 @@ class FusedEncoder:
 
     @property
     def label(self) -> str:
-        return "int8 FFN+QKV+out_proj, 4 boards/workgroup (gfx950)"
+        fmt = "e4m3" if self.fp8 else "int8"
+        return f"{fmt} FFN+QKV+out_proj, 4 boards/workgroup (gfx950)"
 
     # -- buffers and checks ---------------------------------------------------
 
@@ -335,6 +369,7 @@ class FusedEncoder:
         a.policy, a.promo, a.value = policy.data_ptr(), promo.data_ptr(), value.data_ptr()
         a.best_move = best.data_ptr() if (best is not None and mask is not None) else None
         a.out_fp32 = 1 if policy.dtype is torch.float32 else 0
+        a.quant = 1 if self.fp8 else 0
         need = self._lib.bf_workspace_bytes(C.byref(self._shape), a.n)
         if getattr(self, "workspace", None) is None or self.workspace.numel() < need:
             self.workspace = torch.empty(need, device=self.device, dtype=torch.uint8)
@@ -446,6 +481,8 @@ class FusedEncoder:
                      layer_end: Optional[int] = None, want=None):
         """Run with intermediate outputs.  Returns a dict of fresh fp32-output tensors:
         policy, promo, value, [best], plus the taps named in ``want`` (default: all).
+        With ``fp8=True`` the operand taps come back as float8_e4m3fn and the accumulator
+        taps as float32.
 
         ``x_in`` ([n,32,d] fp32) replaces the embedding as the residual stream entering
         layer ``layer_begin``; layers ``[layer_begin, layer_end)`` run, then the heads.
@@ -485,4 +522,10 @@ class FusedEncoder:
                               mask.contiguous() if mask is not None else None,
                               out["policy"], out["promo"], out["value"], best, taps))
         torch.cuda.current_stream(dev).synchronize()   # taps/x_in must outlive the launch
+        if self.fp8:   # the accumulators are fp32 and the operand bytes e4m3 in this format
+            for k in want:
+                if k.startswith("acc_"):
+                    out[k] = out[k].view(torch.float32)
+                elif k.startswith("qa_"):
+                    out[k] = out[k].view(torch.float8_e4m3fn)
         return out

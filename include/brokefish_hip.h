@@ -29,6 +29,11 @@ enum bf_status {
     BF_ERR_DEVICE = -4      /* not a gfx950 device */
 };
 
+enum bf_quant {
+    BF_QUANT_INT8 = 0,
+    BF_QUANT_E4M3 = 1
+};
+
 /* Sizes of one 32-token position, fixed by the position format
  * (reference docs/reference/spec.md:94-106). */
 #define BF_TOKENS 32
@@ -98,6 +103,11 @@ typedef struct {
     float* value;
     int32_t* best_move;
     int32_t out_fp32;
+    /* operand format of the four weight matmuls: BF_QUANT_INT8 (reference
+     * brokefish/nn/quant.py:281-305) or BF_QUANT_E4M3 (quant.py:360-397 with q_max 8,
+     * 256-deep k-tiles and 128-row weight blocks, quant.py:82-105).  The parameter blobs
+     * must have been packed for the same format. */
+    int32_t quant;
     void* workspace;        /* bf_workspace_bytes(shape, n) bytes of device memory */
     size_t workspace_bytes;
     const bf_taps* taps; /* NULL in production */
@@ -111,6 +121,11 @@ int bf_model_forward(const bf_eval_args* args, void* stream);
 /* Quantisation maxima of the signed / unsigned activation formats, for the host to pin
  * against its own constants.  Replaces int8_q_max (reference csrc/encoder.cu:1926-1929). */
 void bf_int8_q_max(double* s8, double* u8);
+
+/* The value a row's (and a weight block's) largest magnitude is mapped to in the e4m3
+ * format.  Replaces fp8_q_max (reference csrc/encoder.cu:1905-1930; pinned against
+ * brokefish/nn/quant.py:105). */
+double bf_fp8_q_max(void);
 
 /* Message for the last non-zero status returned to this thread. */
 const char* bf_last_error(void);

@@ -1,7 +1,8 @@
 """TEST INFRASTRUCTURE -- NOT PRODUCT CODE.
 
 A CPU restatement, in plain PyTorch library calls, of the reference network forward in
-its two modes: fp32, and the int8-simulated forward the HIP evaluator must reproduce.
+its modes: fp32, the int8-simulated forward the HIP evaluator must reproduce, and the
+e4m3-simulated forward of its fp8 variant.
 Only ``tests/``, ``__graft_entry__.smoke()`` and ``bench.py``'s CPU-baseline leg import
 this module; nothing under ``brokefish_amd/`` does.
 
@@ -16,6 +17,9 @@ What each function follows (paths inside the reference tree):
 * :func:`quantise_activations_int8`             -- brokefish/nn/quant.py:246-260
 * :func:`quantise_weights_int8`                 -- brokefish/nn/quant.py:263-278
 * :func:`int8_linear`                           -- brokefish/nn/quant.py:281-305
+* :func:`quantise_activations_e4m3`, :func:`quantise_weights_e4m3`, :func:`fp8_linear`
+                                                -- brokefish/nn/quant.py:161-224, :360-397 with the
+  shipped constants q_max = 8 (:105), tile_k = 256 (:92), block_n = 128 (:82), fp32 accumulator
 * :func:`forward` block structure               -- torch ``TransformerEncoderLayer(norm_first=True)``
   as constructed at brokefish/nn/model.py:303-311 and called at :525 with
   ``src_key_padding_mask=~alive``; the four matmuls routed through ``int8_linear`` and
@@ -40,6 +44,9 @@ ROW_K = 256      # brokefish/nn/quant.py:92
 BLOCK_N = 128    # brokefish/nn/quant.py:82
 Q_MAX_S8 = 127.0  # brokefish/nn/quant.py:237
 Q_MAX_U8 = 255.0  # brokefish/nn/quant.py:241
+Q_MAX_E4M3 = 8.0  # brokefish/nn/quant.py:105
+E4M3_MAX = 448.0  # brokefish/nn/quant.py:73
+E4M3 = torch.float8_e4m3fn   # OCP e4m3: no infinities, maximum 448 (brokefish/nn/quant.py:69-73)
 KING_WHITE, KING_BLACK = 15, 31
 
 
@@ -117,9 +124,69 @@ def int8_linear(x, w, bias, unsigned: bool = False, taps: Optional[dict] = None,
     return y.reshape(*lead, n)
 
 
+def _to_e4m3(x: torch.Tensor) -> torch.Tensor:
+    """Round to e4m3 and back to fp32; clamped first because the format has no infinity."""
+    return x.clamp(-E4M3_MAX, E4M3_MAX).to(E4M3).to(torch.float32)
+
+
+def quantise_activations_e4m3(x: torch.Tensor, q_max: float = Q_MAX_E4M3, tile_k: int = ROW_K):
+    """[M, K] fp32 -> (e4m3-valued fp32 [M, K], scale [M, K // tile_k]); one scale per row
+    per k-tile, the tile's largest magnitude landing on ``q_max``."""
+    m, k = x.shape
+    if k % tile_k:
+        raise ValueError(f"K = {k} is not a multiple of the {tile_k}-element tile")
+    tiles = x.view(m, k // tile_k, tile_k)
+    amax = tiles.abs().amax(dim=-1, keepdim=True)
+    s = torch.where(amax > 0, amax / q_max, torch.ones_like(amax))
+    return _to_e4m3(tiles / s).view(m, k), s.squeeze(-1)
+
+
+def quantise_weights_e4m3(w: torch.Tensor, q_max: float = Q_MAX_E4M3, tile_k: int = ROW_K,
+                          block_n: int = BLOCK_N):
+    """[N, K] fp32 -> (e4m3-valued fp32 [N, K], scale [N // block_n, K // tile_k])."""
+    n, k = w.shape
+    if n % block_n or k % tile_k:
+        raise ValueError(f"weight {tuple(w.shape)} does not tile into {block_n}x{tile_k} blocks")
+    blocks = w.view(n // block_n, block_n, k // tile_k, tile_k)
+    amax = blocks.abs().amax(dim=(1, 3), keepdim=True)
+    s = torch.where(amax > 0, amax / q_max, torch.ones_like(amax))
+    return _to_e4m3(blocks / s).view(n, k), s.reshape(n // block_n, k // tile_k)
+
+
+def fp8_linear(x, w, bias, taps: Optional[dict] = None, name: str = "", q_max: float = Q_MAX_E4M3,
+               tile_k: int = ROW_K, block_n: int = BLOCK_N):
+    """``F.linear`` with both operands e4m3: the product inside one k-tile in fp32, one
+    descale ``* sa * sw`` per tile, fp32 sum over the tiles, then the bias."""
+    lead = x.shape[:-1]
+    a = x.reshape(-1, x.shape[-1]).float()
+    wf = w.float()
+    m, k = a.shape
+    n = wf.shape[0]
+    aq, sa = quantise_activations_e4m3(a, q_max, tile_k)
+    wq, sw = quantise_weights_e4m3(wf, q_max, tile_k, block_n)
+    out = torch.zeros((m, n), dtype=torch.float32)
+    accs = []
+    for t, lo in enumerate(range(0, k, tile_k)):
+        part = aq[:, lo:lo + tile_k] @ wq[:, lo:lo + tile_k].T
+        if taps is not None:
+            accs.append(part.clone())
+        part = part * sa[:, t:t + 1]
+        part = part * sw[:, t].repeat_interleave(block_n)[None, :]
+        out += part
+    if taps is not None:
+        taps.setdefault("qa_" + name, []).append(aq.clone())
+        taps.setdefault("sa_" + name, []).append(sa.clone())
+        taps.setdefault("acc_" + name, []).append(torch.stack(accs))
+    if bias is not None:
+        out = out + bias.float()
+    return out.reshape(*lead, n).to(x.dtype)
+
+
 def _linear(x, w, b, mode, unsigned=False, taps=None, name=""):
     if mode == "int8":
         return int8_linear(x, w, b, unsigned, taps, name)
+    if mode == "e4m3":
+        return fp8_linear(x, w, b, taps, name)
     return F.linear(x, w, b)
 
 
@@ -132,16 +199,22 @@ def n_layers_of(sd) -> int:
 
 def forward(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8",
             mask: Optional[torch.Tensor] = None, n_heads: Optional[int] = None,
-            eps: float = 1e-5, taps: Optional[dict] = None):
+            eps: float = 1e-5, taps: Optional[dict] = None,
+            x_in: Optional[torch.Tensor] = None, layer_begin: int = 0,
+            layer_end: Optional[int] = None):
     """(policy [N,32,64], promo [N,32,4], value [N]) in fp32, plus ``best`` [N] int64
     (slot*64+square of the masked argmax) when ``mask`` is given.
 
-    ``mode`` is ``"fp32"`` (every matmul an ordinary ``F.linear``) or ``"int8"`` (the
-    four body matmuls of every layer through :func:`int8_linear`).
+    ``mode`` is ``"fp32"`` (every matmul an ordinary ``F.linear``), ``"int8"`` (the four
+    body matmuls of every layer through :func:`int8_linear`) or ``"e4m3"`` (through
+    :func:`fp8_linear`).  ``x_in`` replaces the embedding as the residual stream entering
+    layer ``layer_begin``; layers ``[layer_begin, layer_end)`` run (teacher forcing).
     """
-    if mode not in ("fp32", "int8"):
+    if mode not in ("fp32", "int8", "e4m3"):
         raise ValueError(mode)
     x, alive = embed(sd, boards, control, rep)
+    if x_in is not None:
+        x = x_in.clone()
     n, t, d = x.shape
     heads = n_heads if n_heads is not None else d // 32
     dh = d // heads
@@ -149,7 +222,7 @@ def forward(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8
         taps["embed"] = x.clone()
     key_bias = torch.zeros(n, 1, 1, t)
     key_bias.masked_fill_(~alive[:, None, None, :], float("-inf"))
-    for i in range(n_layers_of(sd)):
+    for i in range(layer_begin, n_layers_of(sd) if layer_end is None else layer_end):
         p = f"encoder.layers.{i}."
         y = F.layer_norm(x, (d,), sd[p + "norm1.weight"], sd[p + "norm1.bias"], eps)
         qkv = _linear(y, sd[p + "self_attn.in_proj_weight"], sd[p + "self_attn.in_proj_bias"],
@@ -192,8 +265,8 @@ def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mod
     ``nn.TransformerEncoder`` / ``nn.MultiheadAttention`` modules, exactly the modules the
     reference model is built from (brokefish/nn/model.py:303-311).
 
-    In ``"int8"`` mode the four body matmuls of every layer are diverted to
-    :func:`int8_linear` by intercepting ``torch.nn.functional.linear`` for precisely those
+    In ``"int8"`` (``"e4m3"``) mode the four body matmuls of every layer are diverted to
+    :func:`int8_linear` (:func:`fp8_linear`) by intercepting ``torch.nn.functional.linear`` for precisely those
     weight tensors (the only hook torch's attention module offers for its packed QKV and
     output projections), with the attention fast path switched off so the module really
     calls ``F.linear``; ``linear2`` gets the unsigned quantiser.  Under the torch version
@@ -222,13 +295,15 @@ def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mod
 
     def routed(inp, weight, bias=None):
         u = unsigned_of.get(id(weight))
-        if u is None or mode != "int8":
+        if u is None or mode == "fp32":
             return plain_linear(inp, weight, bias)
         hits[0] += 1
+        if mode == "e4m3":
+            return fp8_linear(inp, weight, bias)
         return int8_linear(inp, weight, bias, unsigned=u)
 
     fast = torch.backends.mha.get_fastpath_enabled()
-    if mode == "int8":
+    if mode != "fp32":
         torch.backends.mha.set_fastpath_enabled(False)
     F.linear = routed
     try:
@@ -237,7 +312,7 @@ def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mod
     finally:
         F.linear = plain_linear
         torch.backends.mha.set_fastpath_enabled(fast)
-    if mode == "int8" and hits[0] != 4 * n_layers:
+    if mode != "fp32" and hits[0] != 4 * n_layers:
         raise AssertionError(f"{hits[0]} matmuls were diverted, expected {4 * n_layers}")
     h = F.layer_norm(h, (d,), sd["norm_f.weight"], sd["norm_f.bias"], eps)
     policy = plain_linear(h, sd["policy.weight"])

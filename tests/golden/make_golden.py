@@ -1,4 +1,5 @@
-"""Writes tests/golden/reference_vectors.npz by running the reference's own Python.
+"""Writes tests/golden/reference_vectors.npz and reference_vectors_e4m3.npz by running the
+reference's own Python.
 
 Run in the build container only (the reference tree is not present anywhere else):
 
@@ -16,6 +17,13 @@ What it records, and why these need the reference itself rather than a closed fo
   whose weights are filled by the formula in :func:`fill_state_dict` (independent of any
   RNG stream) and on eight build-defined positions, plus the layer-0 inputs of the first
   patched matmul.
+
+* the e4m3 twins (second file): ``fp8_linear`` (quant.py:360-397), ``quantise_activations``
+  (:172-188) and ``quantise_weights_bytes`` (:208-224) on the same inputs with the shipped
+  constants (q_max 8, 256-deep tiles, 128-row blocks) and once with the module defaults'
+  128-deep tiles at q_max 448, and the end-to-end forward under
+  ``emulated_forward(net, QuantConfig(weights=True, activations=True, q_max=8, tile_k=256))``.
+  torch's fp32 matmul fixes the summation order inside a k-tile, which no closed form gives.
 
 Inputs are regenerated from the formulas below by the tests; only outputs are stored.
 """
@@ -108,7 +116,18 @@ def main() -> int:
     from brokefish.nn.model import BrokefishNet as RefNet     # noqa: E402
 
     out = {}
+    f8 = {}
+    shipped = rq.QuantConfig(weights=True, activations=True, q_max=rq.Q_MAX, tile_k=rq.ROW_K, block_n=rq.BLOCK_N)
+    wide = rq.QuantConfig(weights=True, activations=True, q_max=448.0)      # module defaults: 128-deep tiles
     for name, x, w, bias, unsigned in linear_cases():
+        f8[f"lin_{name}"] = rq.fp8_linear(x, w, bias, shipped).numpy()
+        f8[f"lin128_{name}"] = rq.fp8_linear(x, w, bias, wide).numpy()
+        qb, ws = rq.quantise_weights_bytes(w, rq.Q_MAX, tile_k=rq.ROW_K)
+        f8[f"wqsum_{name}"] = weight_checksum(qb.numpy())
+        f8[f"ws_{name}"] = ws.numpy()
+        q, s = rq.quantise_activations(x[:, :256].contiguous(), rq.Q_MAX, rq.ROW_K)
+        f8[f"qa_{name}"] = q.to(rq.E4M3).view(torch.uint8).numpy()
+        f8[f"sa_{name}"] = s.numpy()
         y = rq.int8_linear(x, w, bias, unsigned=unsigned)
         out[f"lin_{name}"] = y.numpy()
         qb, ws = rq.quantise_weights_int8_bytes(w)
@@ -131,6 +150,9 @@ def main() -> int:
             p32, q32, v32 = net(boards, control, rep)
             handle.remove()
             p8, q8, v8 = rq.emulated_forward(net, rq.QuantConfig(fmt="int8"))(boards, control, rep)
+            if n_value == 1:
+                pf, qf, vf = rq.emulated_forward(net, shipped)(boards, control, rep)
+                f8["e4m3_policy_nv1"], f8["e4m3_promo_nv1"], f8["e4m3_value_nv1"] = pf.numpy(), qf.numpy(), vf.numpy()
         tag = f"nv{n_value}"
         out[f"fp32_policy_{tag}"], out[f"fp32_promo_{tag}"], out[f"fp32_value_{tag}"] = p32.numpy(), q32.numpy(), v32.numpy()
         out[f"int8_policy_{tag}"], out[f"int8_promo_{tag}"], out[f"int8_value_{tag}"] = p8.numpy(), q8.numpy(), v8.numpy()
@@ -140,6 +162,10 @@ def main() -> int:
     path = os.path.join(HERE, "reference_vectors.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, {k: getattr(v, "shape", None) for k, v in out.items()})
+    f8["torch_version"] = np.array(torch.__version__)
+    path = os.path.join(HERE, "reference_vectors_e4m3.npz")
+    np.savez_compressed(path, **f8)
+    print("wrote", path, {k: getattr(v, "shape", None) for k, v in f8.items()})
     return 0
 
 

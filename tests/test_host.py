@@ -92,9 +92,10 @@ def test_pack_network_layout_and_sizes():
     q2, s2 = hip_impl.quantise_weights_int8(sd["encoder.layers.1.linear2.weight"])
     wsum = l1[9 * 256 + 1024: 9 * 256 + 1024 + 4 * 256].view(np.int32).reshape(4, 256)
     assert (wsum[2] == 128 * q2[:, 512:768].astype(np.int32).sum(1)).all()
-    sw = l1[9 * 256 + 1024 + 4 * 256:9 * 256 + 1024 + 4 * 256 + 20]
-    assert (l1[9 * 256 + 1024 + 4 * 256 + 20:] == 0).all()
-    assert (sw[16:18] == s2).all()
+    sw = l1[9 * 256 + 1024 + 4 * 256:9 * 256 + 1024 + 4 * 256 + 24]
+    assert (l1[9 * 256 + 1024 + 4 * 256 + 24:] == 0).all()
+    # one ffn2 entry per (128-row block, k-chunk); the int8 scale covers the whole reduction
+    assert (sw[16:24] == np.repeat(s2, 4)).all()
     assert (fp[2 * layer_floats:2 * layer_floats + 64 * 256] == sd["emb_square.weight"].numpy().reshape(-1)).all()
     # second block of layer 0 is the K tile of head 0: rows 256..287 of in_proj
     q_qkv, _ = hip_impl.quantise_weights_int8(sd["encoder.layers.0.self_attn.in_proj_weight"])
@@ -125,10 +126,10 @@ def test_registry_and_input_checks():
 def test_constructor_rejections_do_not_need_a_gpu():
     net = BrokefishNet(n_layers=1)
     cls = hip_impl.FusedEncoder
+    with pytest.raises(ValueError):
+        cls(net, fp8=True, int8=True)                    # both quantise the same matmuls
     with pytest.raises(NotImplementedError):
-        cls(net, fp8=True)
-    with pytest.raises(NotImplementedError):
-        cls(net, int8=False)
+        cls(net, int8=False)                             # the unquantised fp16 evaluator is not carried
     with pytest.raises(ValueError):
         cls(net, acc_dtype="bf16")
     with pytest.raises(ValueError):
@@ -138,6 +139,8 @@ def test_constructor_rejections_do_not_need_a_gpu():
     if not torch.cuda.is_available():
         with pytest.raises(RuntimeError, match="no GPU"):
             cls(net, int8=True)
+        with pytest.raises(RuntimeError, match="no GPU"):
+            cls(net, fp8=True)
 
 
 def test_net_matches_reference_parameter_count_and_keys():
