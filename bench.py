@@ -22,15 +22,15 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 OPS_PER_EVAL = 402_653_184            # 2 * 32 tokens * 8 layers * 12 * 256^2 int8 ops in the weight GEMMs
-PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s
+PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s (dense fp8 MFMA: the same figure)
 # HBM bytes per launch of the default workload (batch 4096), from the FETCH_SIZE / WRITE_SIZE
 # counter runs summarised in profiles/eval_kernel_int8_batch4096.md (calibrated on a 1 GiB copy).
 MEASURED_TRAFFIC_BYTES = {4096: 3.07e9}
 
 
-def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0):
-    """The int8-simulated forward of oracle/emulated.py on the host cores (a port, not the
-    reference's files, which do not travel)."""
+def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0, mode: str = "int8"):
+    """The int8- (or e4m3-) simulated forward of oracle/emulated.py on the host cores (a port,
+    not the reference's files, which do not travel)."""
     import torch
     from brokefish_amd import positions
     from oracle import emulated
@@ -39,18 +39,18 @@ def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0):
     torch.set_num_threads(threads)
     with torch.no_grad():
         t0 = time.perf_counter()
-        emulated.forward(sd, b, c, r, mode="int8", mask=m)             # warm-up, also sizes the loop
+        emulated.forward(sd, b, c, r, mode=mode, mask=m)               # warm-up, also sizes the loop
         one = time.perf_counter() - t0
         reps = max(2, min(20, int(budget_s / max(one, 1e-3))))
         times = []
         for _ in range(reps):
             t0 = time.perf_counter()
-            emulated.forward(sd, b, c, r, mode="int8", mask=m)
+            emulated.forward(sd, b, c, r, mode=mode, mask=m)
             times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
     return {"value": batch / med, "unit": "evals/s", "cores": threads, "kind": "port",
-            "sample": f"{reps} reps of batch {batch} (int8-simulated PyTorch forward, median), "
+            "sample": f"{reps} reps of batch {batch} ({mode}-simulated PyTorch forward, median), "
                       f"os.cpu_count()={os.cpu_count()}"}
 
 
@@ -60,6 +60,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=4096)
+    ap.add_argument("--quant", choices=("int8", "e4m3"), default="int8",
+                    help="operand format of the weight matmuls; int8 is the headline metric, e4m3 the fp8 variant")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=64)
     ap.add_argument("--sweep", action="store_true",
@@ -79,7 +81,8 @@ def main() -> int:
 
     torch.manual_seed(0)
     net = BrokefishNet().eval()                                  # seed-0 random init, reference init rules
-    model = encoder_impl("hip")(net, int8=True)                  # fp16 logits: the search contract
+    fp8 = a.quant == "e4m3"
+    model = encoder_impl("hip")(net, fp8=True) if fp8 else encoder_impl("hip")(net, int8=True)   # fp16 logits: the search contract
     b, c, r, m = positions.random_positions(a.batch, plies=120, seed=0)
     bd, cd, rd, md = b.cuda(), c.cuda(), r.cuda(), m.cuda()
 
@@ -103,16 +106,16 @@ def main() -> int:
     kern_ms = model.time_kernel_ms(bd, cd, rd, md, warmup=3, iters=max(a.steps, 10))
     achieved = OPS_PER_EVAL * a.batch / (kern_ms * 1e-3) / 1e12
     line = {
-        "metric": "network evals/sec at batch 4096 int8 on 1 MI355X",
+        "metric": f"network evals/sec at batch 4096 {'fp8 e4m3' if fp8 else 'int8'} on 1 MI355X",
         "value": evals, "unit": "evals/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8", "data": "synthetic",
-        "config": {"workload": f"configs[1]: 8-layer d256 8-head FFN1024 int8 evaluator, batch {a.batch}, "
+        "dtype": "fp8" if fp8 else "int8", "data": "synthetic",
+        "config": {"workload": f"configs[{4 if fp8 else 1}]: 8-layer d256 8-head FFN1024 {a.quant} evaluator, batch {a.batch}, "
                                "seeded random playouts 0-120 plies, legal-move mask ANDed in-kernel, "
                                "fp16 logits out, seed-0 random-init weights"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
                      "frac": achieved / (PEAK_INT8_OPS / 1e12),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(a.batch),
+                     "traffic": None if fp8 else MEASURED_TRAFFIC_BYTES.get(a.batch),
                      "kernel_ms": kern_ms, "ops_per_launch": OPS_PER_EVAL * a.batch},
     }
     if a.sweep:
@@ -126,7 +129,7 @@ def main() -> int:
         line["sweep"] = pts
     if not a.no_cpu:
         threads = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
-        line["cpu_baseline"] = cpu_baseline(net, a.cpu_batch, threads)
+        line["cpu_baseline"] = cpu_baseline(net, a.cpu_batch, threads, mode=a.quant)
     print(json.dumps(line))
     return 0
 

@@ -163,7 +163,9 @@ const char* bf_profile_phase_name(int i);
  *     out-proj tiles 0..7
  *     ffn1 tiles 0..31
  *     for ffn2 output tile n: for k-chunk c = 0..3: block (n, c)
- * and after the last layer three 32 KiB fp32 head tiles: head tile m (rows 32m..32m+31
+ * In the e4m3 format the bytes are OCP e4m3 codes instead of int8 values, in the same
+ * order; each weight scale then covers a 128-row x 256-deep block, wsum is all zero.
+ * After the last layer three 32 KiB fp32 head tiles: head tile m (rows 32m..32m+31
  * of [policy(64); promo(4); value(n_value); zeros]), fragment (n, q), lane 32g + o holds
  * the four floats W[32 m + o][32 n + 8 q + 4 g + 0..3].
  *
@@ -172,7 +174,9 @@ const char* bf_profile_phase_name(int i);
  * in 4 KiB passes):
  *     ln1_gamma[d] ln1_beta[d] b_qkv[3d] b_out[d] ln2_gamma[d] ln2_beta[d] b_ffn1[f]
  *     b_ffn2[d] wsum[kc_f][d] (int32: 128 * sum of the int8 weights of ffn2 row over
- *     k-chunk c) sw_qkv[3d/128] sw_out[d/128] sw_ffn1[f/128] sw_ffn2[d/128]
+ *     k-chunk c) sw_qkv[3d/128] sw_out[d/128] sw_ffn1[f/128] sw_ffn2[d/128][kc_f]
+ *     (weight scales per 128 output rows; ffn2 carries one per k-chunk, which the int8
+ *     format fills with the same value four times)
  * then the five embedding tables (square 64, type_special 12, color_turn 4, clock 101,
  * rep 3 rows of d) and norm_f gamma[d], beta[d].
  * ----------------------------------------------------------------------------------- */

@@ -26,7 +26,7 @@ def test_library_loads_and_exports_every_declared_symbol():
     names = _declared_functions()
     assert {"bf_model_forward", "bf_wstream_bytes", "bf_fparams_floats", "bf_int8_q_max",
             "bf_last_error", "bf_time_kernel_ms", "bf_layer_stride_floats", "bf_workspace_bytes",
-            "bf_profile_phases", "bf_profile_phase_count", "bf_profile_phase_name"} <= set(names)
+            "bf_profile_phases", "bf_profile_phase_count", "bf_profile_phase_name", "bf_fp8_q_max"} <= set(names)
     for n in names:
         assert hasattr(lib, n), f"{n} is declared in include/brokefish_hip.h but not exported"
 
@@ -34,6 +34,7 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_constants_agree_between_host_and_library():
     # the counterpart of the reference's Python<->CUDA constant pin (tests/test_quant.py:233-269)
     assert hip_impl.int8_q_max() == (hip_impl.Q_MAX_S8, hip_impl.Q_MAX_U8) == (127.0, 255.0)
+    assert hip_impl.fp8_q_max() == hip_impl.Q_MAX_E4M3 == 8.0
     lib = hip_impl.load_library()
     shape = hip_impl._Shape(256, 8, 8, 1024, 1, 1e-5)
     assert lib.bf_wstream_bytes(ctypes.byref(shape)) == (8 * 24 + 3) * 32768
