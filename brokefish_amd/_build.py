@@ -20,7 +20,9 @@ HIP_LIB = os.path.join(HERE, "libbrokefish_hip.so")
 CHESSGEN_LIB = os.path.join(HERE, "libbf_chessgen.so")
 
 HIP_SOURCES = ["bf_host.hip", "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip",
-               "bf_variant_prod_fp8.hip", "bf_variant_taps_fp8.hip"]
+               "bf_variant_prod_fp8.hip", "bf_variant_taps_fp8.hip",
+               "bf_variant_board256.hip", "bf_variant_board256_taps.hip",
+               "bf_variant_board512.hip", "bf_variant_board512_taps.hip"]
 # -ffp-contract=off: the kernel's fp32 arithmetic is specified operation by operation
 # (fused multiply-adds are written explicitly), so the compiler must not fuse on its own.
 # The packed-fp32 feature is disabled so no v_pk_*_f32 instructions are generated.
@@ -64,7 +66,7 @@ def build_hip(verbose: bool = False, extra=()) -> str:
             print(r.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=len(HIP_SOURCES)) as pool:
+    with ThreadPoolExecutor(max_workers=min(len(HIP_SOURCES), os.cpu_count() or 4)) as pool:
         objs = list(pool.map(compile_one, HIP_SOURCES))
     _run([hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB] + objs)
     return HIP_LIB

@@ -18,7 +18,8 @@
 //
 // Arithmetic contract (what the CPU checker restates operation by operation):
 //   embedding  ((sq + ts) + ct) + (clock + rep)                        fp32
-//   LayerNorm  two partial sums per row (one per lane half), sequential over tiles then r
+//   LayerNorm  per lane half four group sums (a quarter of the tiles each, sequential over
+//              tiles then r) added in group order, then the two halves
 //   quantise   s = amax / qmax, q = rint(x / s)  (x / s as a correctly rounded quotient)
 //   GEMM       exact int32; descale fl(fl(acc * sa) * sw) + b; several k-chunks are summed
 //              in fp64 before the single cast to fp32
@@ -68,6 +69,27 @@ constexpr int G_SQ = 0, G_TS = 64 * D, G_CT = G_TS + 12 * D, G_CLOCK = G_CT + 4 
               G_REP = G_CLOCK + 101 * D, G_NFG = G_REP + 3 * D, G_NFB = G_NFG + D,
               GLOBAL_FLOATS = G_NFB + D;
 
+// Layout of the one-position-per-workgroup kernel (bf_board.hip.h), for model width DM: wave w
+// owns tiles TW*w .. TW*w+TW-1 of the width.  Per layer a wave streams BPW weight blocks in its
+// own consumption order and reads PW_FLOATS side parameters (part A: attention phase, part B:
+// feed-forward phase); see include/brokefish_hip.h for the blob layouts.
+template <int DM>
+struct Layout {
+    static constexpr int D = DM, F = 4 * DM, NT = DM / 32, TW = NT / 4, CW = 32 * TW, KC = DM / 256,
+                         KCF = F / 256, HALVES = F / 1024;
+    static constexpr int BPW = 3 * TW * KC + TW * KC + HALVES * (8 * KC + 4 * TW);
+    static constexpr int HB = NT / 2;              // head blocks per wave (8 fp32 fragments each)
+    static constexpr int SLOTS = DM == 256 ? 3 : 2;  // depth of a wave's private weight ring, in blocks
+    static constexpr int A_LN1G = 0, A_LN1B = CW, A_BQ = 2 * CW, A_BK = 3 * CW, A_BV = 4 * CW, A_BOUT = 5 * CW,
+                         A_SW = 6 * CW, A_FLOATS = 6 * CW + 16;
+    static constexpr int B_LN2G = 0, B_LN2B = CW, B_BFF1 = 2 * CW, B_BFF2 = 2 * CW + 256 * HALVES,
+                         B_WSUM = 3 * CW + 256 * HALVES, B_SW = B_WSUM + KCF * CW, B_FLOATS = B_SW + 32;
+    static constexpr int PW_FLOATS = A_FLOATS + B_FLOATS;
+    static constexpr int G_SQ = 0, G_TS = 64 * D, G_CT = G_TS + 12 * D, G_CLOCK = G_CT + 4 * D,
+                         G_REP = G_CLOCK + 101 * D, G_NFG = G_REP + 3 * D, G_NFB = G_NFG + D,
+                         GLOBAL_FLOATS = G_NFB + D;
+};
+
 constexpr int N_PHASES = 12;
 // phase slots of the optional cycle profile
 enum { PH_EMBED, PH_LN1, PH_QKV, PH_ATTN, PH_OUT, PH_LN2, PH_FF1, PH_FF2, PH_HEADS, PH_STORE, PH_SYNC, PH_TOTAL };
@@ -98,5 +120,10 @@ hipError_t launch_taps(const KArgs& k, int grid, hipStream_t stream);
 hipError_t launch_prof(const KArgs& k, int grid, hipStream_t stream);
 hipError_t launch_prod_fp8(const KArgs& k, int grid, hipStream_t stream);
 hipError_t launch_taps_fp8(const KArgs& k, int grid, hipStream_t stream);
+// one position per workgroup (grid = n), int8, for the 256- and the 512-wide network
+hipError_t launch_board256(const KArgs& k, hipStream_t stream);
+hipError_t launch_board256_taps(const KArgs& k, hipStream_t stream);
+hipError_t launch_board512(const KArgs& k, hipStream_t stream);
+hipError_t launch_board512_taps(const KArgs& k, hipStream_t stream);
 
 }  // namespace bf

@@ -15,10 +15,46 @@ static int fail(int code, const char* msg) {
     return code;
 }
 
-static bool shape_ok(const bf_shape* s) {
+static bool shape_ok(const bf_shape* s) {   // the four-positions-per-workgroup kernel
     return s && s->d_model == bf::D && s->d_ff == bf::F && s->n_heads == bf::NH && s->n_layers >= 1 &&
            (s->n_value == 1 || s->n_value == 3);
 }
+
+static bool shape512(const bf_shape* s) {
+    return s && s->d_model == 512 && s->d_ff == 2048 && s->n_heads == 16 && s->n_layers >= 1 &&
+           (s->n_value == 1 || s->n_value == 3);
+}
+
+static bool board_shape_ok(const bf_shape* s) { return shape_ok(s) || shape512(s); }
+
+// AUTO prefers one position per workgroup up to this many positions (256-wide network): below
+// it the four-per-workgroup launch leaves most compute units idle.
+static const int64_t kBoardMaxN = 768;
+
+template <int DM>
+static size_t board_wstream_bytes(int n_layers) {
+    typedef bf::Layout<DM> L;
+    return (size_t)4 * ((size_t)n_layers * L::BPW + L::HB) * bf::BLOCK;
+}
+template <int DM>
+static size_t board_fparams_floats(int n_layers) {
+    typedef bf::Layout<DM> L;
+    return (size_t)4 * n_layers * L::PW_FLOATS + L::GLOBAL_FLOATS;
+}
+
+extern "C" size_t bf_board_wstream_bytes(const bf_shape* s) {
+    if (shape_ok(s)) return board_wstream_bytes<256>(s->n_layers);
+    if (shape512(s)) return board_wstream_bytes<512>(s->n_layers);
+    return 0;
+}
+
+extern "C" size_t bf_board_fparams_floats(const bf_shape* s) {
+    if (shape_ok(s)) return board_fparams_floats<256>(s->n_layers);
+    if (shape512(s)) return board_fparams_floats<512>(s->n_layers);
+    return 0;
+}
+
+extern "C" int64_t bf_board_max_n(void) { return kBoardMaxN; }
 
 extern "C" size_t bf_wstream_bytes(const bf_shape* s) {
     if (!shape_ok(s)) return 0;
@@ -50,29 +86,58 @@ extern "C" double bf_fp8_q_max(void) { return 8.0; }
 
 extern "C" const char* bf_last_error(void) { return g_err; }
 
-static int check_args(const bf_eval_args* a, bf::KArgs* k) {
+// Which kernel runs for these arguments (enum bf_kernel), or a negative status.
+static int choose_kernel(const bf_eval_args* a) {
     if (!a) return fail(BF_ERR_ARGUMENT, "args is NULL");
-    if (!shape_ok(&a->shape))
+    if (!board_shape_ok(&a->shape))
         return fail(BF_ERR_UNSUPPORTED,
-                    "unsupported network shape: this build carries d_model=256, n_heads=8, d_ff=1024, "
-                    "n_layers>=1, n_value in {1,3}");
+                    "unsupported network shape: this build carries d_model=256/n_heads=8/d_ff=1024 and "
+                    "d_model=512/n_heads=16/d_ff=2048, n_layers>=1, n_value in {1,3}");
+    if (a->quant != BF_QUANT_INT8 && a->quant != BF_QUANT_E4M3)
+        return fail(BF_ERR_ARGUMENT, "quant must be BF_QUANT_INT8 or BF_QUANT_E4M3");
+    const bool have_quad = a->wstream && a->fparams, have_board = a->board_wstream && a->board_fparams;
+    const bool quad_can = shape_ok(&a->shape) && have_quad;
+    const bool board_can = have_board && a->quant == BF_QUANT_INT8;
+    switch (a->kernel) {
+    case BF_KERNEL_QUAD:
+        if (!quad_can) return fail(BF_ERR_UNSUPPORTED, "the four-positions-per-workgroup kernel needs the 256-wide network and wstream/fparams");
+        return BF_KERNEL_QUAD;
+    case BF_KERNEL_BOARD:
+        if (!board_can) return fail(BF_ERR_UNSUPPORTED, "the one-position-per-workgroup kernel needs board_wstream/board_fparams and the int8 format");
+        return BF_KERNEL_BOARD;
+    case BF_KERNEL_AUTO:
+        if (board_can && (!quad_can || a->n <= kBoardMaxN)) return BF_KERNEL_BOARD;
+        if (quad_can) return BF_KERNEL_QUAD;
+        return fail(BF_ERR_ARGUMENT, shape512(&a->shape)
+                        ? "the 512-wide network runs on the one-position-per-workgroup kernel: int8, board_wstream/board_fparams required"
+                        : "wstream/fparams must not be NULL");
+    default:
+        return fail(BF_ERR_ARGUMENT, "kernel must be BF_KERNEL_AUTO, BF_KERNEL_QUAD or BF_KERNEL_BOARD");
+    }
+}
+
+extern "C" int bf_kernel_choice(const bf_eval_args* args) { return choose_kernel(args); }
+
+static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
+    *kind = choose_kernel(a);
+    if (*kind < 0) return *kind;
+    const bool board = *kind == BF_KERNEL_BOARD;
     if (a->n < 1 || a->n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
     if (!a->boards || !a->control || !a->rep) return fail(BF_ERR_ARGUMENT, "boards/control/rep must not be NULL");
-    if (!a->wstream || !a->fparams) return fail(BF_ERR_ARGUMENT, "wstream/fparams must not be NULL");
     if (!a->policy || !a->promo || !a->value) return fail(BF_ERR_ARGUMENT, "policy/promo/value must not be NULL");
-    if (((uintptr_t)a->wstream & 15) || ((uintptr_t)a->fparams & 15))
-        return fail(BF_ERR_ARGUMENT, "wstream/fparams must be 16-byte aligned");
+    const uint8_t* ws = board ? a->board_wstream : a->wstream;
+    const float* fp = board ? a->board_fparams : a->fparams;
+    if (((uintptr_t)ws & 15) || ((uintptr_t)fp & 15))
+        return fail(BF_ERR_ARGUMENT, "the parameter blobs must be 16-byte aligned");
     if (((uintptr_t)a->policy & 15) || ((uintptr_t)a->promo & 7) || ((uintptr_t)a->boards & 1))
         return fail(BF_ERR_ARGUMENT, "policy must be 16-byte and promo 8-byte aligned");
     if (a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
-    if (a->quant != BF_QUANT_INT8 && a->quant != BF_QUANT_E4M3)
-        return fail(BF_ERR_ARGUMENT, "quant must be BF_QUANT_INT8 or BF_QUANT_E4M3");
-    if (!a->workspace || ((uintptr_t)a->workspace & 15) || a->workspace_bytes < bf_workspace_bytes(&a->shape, a->n))
+    if (!board && (!a->workspace || ((uintptr_t)a->workspace & 15) || a->workspace_bytes < bf_workspace_bytes(&a->shape, a->n)))
         return fail(BF_ERR_ARGUMENT, "workspace must be 16-byte aligned and hold bf_workspace_bytes(shape, n) bytes");
     memset(k, 0, sizeof(*k));
     k->boards = a->boards; k->control = a->control; k->rep = a->rep; k->mask = a->mask;
     k->n = (int)a->n;
-    k->wstream = a->wstream; k->fparams = a->fparams;
+    k->wstream = ws; k->fparams = fp;
     k->policy = a->policy; k->promo = a->promo; k->value = a->value; k->best = a->best_move;
     k->out_fp32 = a->out_fp32 ? 1 : 0;
     k->xpark = static_cast<float*>(a->workspace);
@@ -90,10 +155,16 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k) {
     return BF_OK;
 }
 
-static int launch(const bf_eval_args* a, const bf::KArgs& k, hipStream_t stream) {
+static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream_t stream) {
     const int grid = (k.n + bf::WAVES - 1) / bf::WAVES;
     hipError_t e;
-    if (a->quant == BF_QUANT_E4M3)
+    if (kind == BF_KERNEL_BOARD) {
+        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
+        if (a->shape.d_model == 512)
+            e = a->taps ? bf::launch_board512_taps(k, stream) : bf::launch_board512(k, stream);
+        else
+            e = a->taps ? bf::launch_board256_taps(k, stream) : bf::launch_board256(k, stream);
+    } else if (a->quant == BF_QUANT_E4M3)
         e = a->taps ? bf::launch_taps_fp8(k, grid, stream) : bf::launch_prod_fp8(k, grid, stream);
     else
         e = k.profile ? bf::launch_prof(k, grid, stream)
@@ -108,20 +179,22 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, hipStream_t stream)
 
 extern "C" int bf_model_forward(const bf_eval_args* args, void* stream) {
     bf::KArgs k;
-    const int rc = check_args(args, &k);
+    int kind;
+    const int rc = check_args(args, &k, &kind);
     if (rc) return rc;
-    return launch(args, k, (hipStream_t)stream);
+    return launch(args, k, kind, (hipStream_t)stream);
 }
 
 extern "C" int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_t* cycles) {
     bf::KArgs k;
-    const int rc = check_args(args, &k);
+    int kind;
+    const int rc = check_args(args, &k, &kind);
     if (rc) return rc;
     if (args->taps) return fail(BF_ERR_ARGUMENT, "the phase profile runs without taps");
     if (args->quant != BF_QUANT_INT8) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the int8 format only");
     if (!cycles) return fail(BF_ERR_ARGUMENT, "cycles must not be NULL");
     k.profile = reinterpret_cast<unsigned long long*>(cycles);
-    return launch(args, k, (hipStream_t)stream);
+    return launch(args, k, kind, (hipStream_t)stream);
 }
 
 extern "C" int bf_profile_phase_count(void) { return bf::N_PHASES; }
@@ -135,16 +208,17 @@ extern "C" const char* bf_profile_phase_name(int i) {
 
 extern "C" double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int iters) {
     bf::KArgs k;
-    int rc = check_args(args, &k);
+    int kind;
+    int rc = check_args(args, &k, &kind);
     if (rc) return rc;
     if (iters < 1 || warmup < 0) return fail(BF_ERR_ARGUMENT, "iters must be >= 1 and warmup >= 0");
     hipStream_t s = (hipStream_t)stream;
     hipEvent_t e0, e1;
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
         return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
-    for (int i = 0; i < warmup && !rc; i++) rc = launch(args, k, s);
+    for (int i = 0; i < warmup && !rc; i++) rc = launch(args, k, kind, s);
     (void)hipEventRecord(e0, s);
-    for (int i = 0; i < iters && !rc; i++) rc = launch(args, k, s);
+    for (int i = 0; i < iters && !rc; i++) rc = launch(args, k, kind, s);
     (void)hipEventRecord(e1, s);
     const hipError_t e = hipEventSynchronize(e1);
     float ms = 0.0f;

@@ -1,0 +1,6 @@
+// Kernel variant "board512" of the evaluator (one position per workgroup), compiled as its own translation unit.
+#include "bf_board.hip.h"
+
+namespace bf {
+hipError_t launch_board512(const KArgs& k, hipStream_t stream) { return board::launch_board<512, false>(k, stream); }
+}  // namespace bf

@@ -57,7 +57,8 @@ class _Args(C.Structure):
                 ("wstream", C.c_void_p), ("fparams", C.c_void_p),
                 ("policy", C.c_void_p), ("promo", C.c_void_p), ("value", C.c_void_p),
                 ("best_move", C.c_void_p), ("out_fp32", C.c_int32), ("quant", C.c_int32),
-                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("taps", C.POINTER(_Taps))]
+                ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("taps", C.POINTER(_Taps)),
+                ("board_wstream", C.c_void_p), ("board_fparams", C.c_void_p), ("kernel", C.c_int32)]
 
 
 _lib = None
@@ -93,6 +94,13 @@ def load_library():
         L.bf_profile_phase_name.argtypes = [C.c_int]
         L.bf_int8_q_max.argtypes = [C.POINTER(C.c_double), C.POINTER(C.c_double)]
         L.bf_fp8_q_max.restype = C.c_double
+        L.bf_board_wstream_bytes.restype = C.c_size_t
+        L.bf_board_wstream_bytes.argtypes = [C.POINTER(_Shape)]
+        L.bf_board_fparams_floats.restype = C.c_size_t
+        L.bf_board_fparams_floats.argtypes = [C.POINTER(_Shape)]
+        L.bf_board_max_n.restype = C.c_int64
+        L.bf_kernel_choice.restype = C.c_int
+        L.bf_kernel_choice.argtypes = [C.POINTER(_Args)]
         _lib = L
     return _lib
 
@@ -233,6 +241,75 @@ def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_v
     return wstream, fparams
 
 
+def pack_network_board(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_value: int):
+    """state_dict -> (board_wstream uint8, board_fparams float32): the int8 network in the order
+    of the one-position-per-workgroup kernel (layout at the end of include/brokefish_hip.h).
+    Wave w owns tiles tw*w .. tw*w+tw-1 of the width; each wave gets its own weight stream and
+    its own slice of the side parameters."""
+    nt, tw, kc, kcf, halves = d // 32, d // 128, d // 256, f // 256, f // 1024
+    cw = 32 * tw
+    get = lambda k: sd[k].detach().float().cpu()
+    quant = []
+    for l in range(n_layers):
+        p = f"encoder.layers.{l}."
+        quant.append([quantise_weights_int8(get(p + nm)) for nm in
+                      ("self_attn.in_proj_weight", "self_attn.out_proj.weight", "linear1.weight", "linear2.weight")])
+    head = np.zeros((128, d), np.float32)
+    head[:N_POLICY] = get("policy.weight").numpy()
+    head[N_POLICY:N_POLICY + N_PROMO] = get("promo.weight").numpy()
+    head[N_POLICY + N_PROMO:N_POLICY + N_PROMO + n_value] = get("value.weight").numpy()
+    stream, fl = [], []
+    for w in range(4):
+        own = slice(cw * w, cw * (w + 1))
+        tiles = [tw * w + i for i in range(tw)]
+        for l in range(n_layers):
+            p = f"encoder.layers.{l}."
+            (q_qkv, s_qkv), (q_out, s_out), (q_ff1, s_ff1), (q_ff2, s_ff2) = quant[l]
+            for n in tiles:
+                for part in range(3):
+                    for c in range(kc):
+                        stream.append(pack_int8_block(q_qkv, part * nt + n, 256 * c))
+            for n in tiles:
+                for c in range(kc):
+                    stream.append(pack_int8_block(q_out, n, 256 * c))
+            for hh in range(halves):
+                for i in range(8):
+                    for c in range(kc):
+                        stream.append(pack_int8_block(q_ff1, 32 * hh + 8 * w + i, 256 * c))
+                for c in range(4 * hh, 4 * hh + 4):
+                    for n in tiles:
+                        stream.append(pack_int8_block(q_ff2, n, 256 * c))
+            b_qkv = get(p + "self_attn.in_proj_bias").numpy()
+            sw_a = np.zeros(16, np.float32)
+            for i, n in enumerate(tiles):
+                sw_a[i] = s_qkv[(32 * n) // BLOCK_N]
+                sw_a[tw + i] = s_qkv[(d + 32 * n) // BLOCK_N]
+                sw_a[2 * tw + i] = s_qkv[(2 * d + 32 * n) // BLOCK_N]
+                sw_a[3 * tw + i] = s_out[(32 * n) // BLOCK_N]
+            part_a = [get(p + "norm1.weight").numpy()[own], get(p + "norm1.bias").numpy()[own],
+                      b_qkv[:d][own], b_qkv[d:2 * d][own], b_qkv[2 * d:][own],
+                      get(p + "self_attn.out_proj.bias").numpy()[own], sw_a]
+            hidden = np.concatenate([np.arange(1024 * hh + 256 * w, 1024 * hh + 256 * w + 256) for hh in range(halves)])
+            wsum = (128 * q_ff2.astype(np.int32).reshape(d, kcf, 256).sum(axis=2)).T[:, own]   # [kcf, cw]
+            sw_b = np.zeros(32, np.float32)
+            for hh in range(halves):
+                for i in range(8):
+                    sw_b[8 * hh + i] = s_ff1[(1024 * hh + 256 * w + 32 * i) // BLOCK_N]
+            for i, n in enumerate(tiles):
+                sw_b[8 * halves + i] = s_ff2[(32 * n) // BLOCK_N]
+            part_b = [get(p + "norm2.weight").numpy()[own], get(p + "norm2.bias").numpy()[own],
+                      get(p + "linear1.bias").numpy()[hidden], get(p + "linear2.bias").numpy()[own],
+                      np.ascontiguousarray(wsum, dtype=np.int32).view(np.float32).reshape(-1), sw_b]
+            fl += part_a + part_b
+        stream.append(pack_head_tile(head, w).view(np.uint8))
+    for name in ("emb_square", "emb_type_special", "emb_color_turn", "emb_clock", "emb_rep"):
+        fl.append(get(name + ".weight").numpy())
+    fl += [get("norm_f.weight").numpy(), get("norm_f.bias").numpy()]
+    wstream = np.concatenate([x.reshape(-1) for x in stream])
+    fparams = np.concatenate([np.ascontiguousarray(x, dtype=np.float32).reshape(-1) for x in fl])
+    return wstream, fparams
+
+
 # --------------------------------------------------------------------------- #
 # the evaluator object
 # --------------------------------------------------------------------------- #
@@ -241,6 +318,8 @@ class FusedEncoder:
     """Boards to logits in one launch (see the module docstring)."""
 
     D, DFF, T, H = 256, 1024, 32, 8
+    SHAPES = ((256, 1024, 8), (512, 2048, 16))     # (d_model, d_ff, heads) the library carries
+    KERNELS = {"auto": 0, "quad": 1, "board": 2}   # enum bf_kernel
     ACC_DTYPES = ("fp16", "fp32")
     n_value = 1
     vmode = 0
@@ -249,7 +328,9 @@ class FusedEncoder:
     def __init__(self, source, acc_dtype: str = "fp16", fp8: bool = False,
                  int8: Optional[bool] = None, two_boards: Optional[bool] = None,
                  int8_scheme: str = "all", out_dtype: torch.dtype = torch.float16,
-                 device: Optional[torch.device] = None):
+                 device: Optional[torch.device] = None, kernel: str = "auto"):
+        if kernel not in self.KERNELS:
+            raise ValueError(f"kernel must be one of {tuple(self.KERNELS)}, got {kernel!r}")
         if acc_dtype not in self.ACC_DTYPES:
             raise ValueError(f"acc_dtype must be one of {self.ACC_DTYPES}, got {acc_dtype!r}")
         if fp8 and int8:
@@ -280,10 +361,17 @@ class FusedEncoder:
         self.d_ff = first.linear1.out_features
         self.d_head = self.d_model // self.n_heads
         self.eps = float(first.norm1.eps)
-        if (self.d_model, self.d_ff, self.n_heads) != (self.D, self.DFF, self.H):
+        if (self.d_model, self.d_ff, self.n_heads) not in self.SHAPES:
             raise ValueError(
-                f"kernel is compiled for d_model={self.D}, d_ff={self.DFF}, heads={self.H}; "
+                f"kernels are compiled for (d_model, d_ff, heads) in {self.SHAPES}; "
                 f"got {self.d_model}, {self.d_ff}, {self.n_heads}")
+        wide = self.d_model != self.D
+        if wide and fp8:
+            raise NotImplementedError("the 512-wide network runs in int8 only")
+        if wide and kernel == "quad":
+            raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernel only")
+        if fp8 and kernel == "board":
+            raise NotImplementedError("the one-position-per-workgroup kernel runs in int8 only")
         if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
             raise ValueError("the evaluator implements pre-norm ReLU layers only")
         self.n_value = int(net.value.weight.shape[0]) if net is not None else 1
@@ -312,20 +400,36 @@ class FusedEncoder:
                                ("emb_clock", 101), ("emb_rep", 3), ("policy", 64), ("promo", 4), ("value", 1)):
                 sd[name + ".weight"] = torch.zeros(rows, d)
             sd["norm_f.weight"], sd["norm_f.bias"] = torch.ones(d), torch.zeros(d)
-        wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value,
-                                        fmt="e4m3" if self.fp8 else "int8")
-        if wstream.size != self._lib.bf_wstream_bytes(C.byref(self._shape)) or \
-                fparams.size != self._lib.bf_fparams_floats(C.byref(self._shape)):
-            raise RuntimeError("packed blob sizes disagree with the library's layout")
-        self.wstream = torch.from_numpy(wstream).to(self.device)
-        self.fparams = torch.from_numpy(fparams).to(self.device)
+        # Two packings of the same weights, one per kernel (see include/brokefish_hip.h): the
+        # four-positions-per-workgroup kernel (256-wide network) and the one-position-per-workgroup
+        # kernel (int8; small launches of the 256-wide network and the 512-wide network).
+        self.kernel = kernel
+        self.wstream = self.fparams = self.board_wstream = self.board_fparams = None
+        if not wide and kernel != "board":
+            wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value,
+                                            fmt="e4m3" if self.fp8 else "int8")
+            if wstream.size != self._lib.bf_wstream_bytes(C.byref(self._shape)) or \
+                    fparams.size != self._lib.bf_fparams_floats(C.byref(self._shape)):
+                raise RuntimeError("packed blob sizes disagree with the library's layout")
+            self.wstream = torch.from_numpy(wstream).to(self.device)
+            self.fparams = torch.from_numpy(fparams).to(self.device)
+        if not self.fp8 and kernel != "quad":
+            wstream, fparams = pack_network_board(sd, self.n_layers, self.d_model, self.d_ff, self.n_value)
+            if wstream.size != self._lib.bf_board_wstream_bytes(C.byref(self._shape)) or \
+                    fparams.size != self._lib.bf_board_fparams_floats(C.byref(self._shape)):
+                raise RuntimeError("packed blob sizes disagree with the library's layout (board kernel)")
+            self.board_wstream = torch.from_numpy(wstream).to(self.device)
+            self.board_fparams = torch.from_numpy(fparams).to(self.device)
         self._buffered_full = 0
         self.best_move = None
 
     @property
     def label(self) -> str:
         fmt = "e4m3" if self.fp8 else "int8"
-        return f"{fmt} FFN+QKV+out_proj, 4 boards/workgroup (gfx950)"
+        per = {"auto": "4 or 1 boards/workgroup by batch size", "quad": "4 boards/workgroup",
+               "board": "1 board/workgroup"}[self.kernel if self.board_wstream is not None and self.wstream is not None
+                                             else ("board" if self.wstream is None else "quad")]
+        return f"{fmt} FFN+QKV+out_proj, {per} (gfx950)"
 
     # -- buffers and checks ---------------------------------------------------
 
@@ -335,7 +439,7 @@ class FusedEncoder:
             self.promo_out = torch.empty(n, T, N_PROMO, device=self.device, dtype=self.out_dtype)
             self.value_out = torch.empty(n, device=self.device, dtype=torch.float32)
             self.best_out = torch.empty(n, device=self.device, dtype=torch.int32)
-            nbytes = self._lib.bf_workspace_bytes(C.byref(self._shape), n)
+            nbytes = self._lib.bf_workspace_bytes(C.byref(self._shape), n) if self.wstream is not None else 0
             self.workspace = torch.empty(nbytes, device=self.device, dtype=torch.uint8)
             self._buffered_full = n
 
@@ -365,17 +469,33 @@ class FusedEncoder:
         a.mask = mask.data_ptr() if mask is not None else None
         a.n = boards.shape[0]
         a.shape = self._shape
-        a.wstream, a.fparams = self.wstream.data_ptr(), self.fparams.data_ptr()
+        if self.wstream is not None:
+            a.wstream, a.fparams = self.wstream.data_ptr(), self.fparams.data_ptr()
+        if self.board_wstream is not None:
+            a.board_wstream, a.board_fparams = self.board_wstream.data_ptr(), self.board_fparams.data_ptr()
+        a.kernel = self.KERNELS[self.kernel]
         a.policy, a.promo, a.value = policy.data_ptr(), promo.data_ptr(), value.data_ptr()
         a.best_move = best.data_ptr() if (best is not None and mask is not None) else None
         a.out_fp32 = 1 if policy.dtype is torch.float32 else 0
         a.quant = 1 if self.fp8 else 0
-        need = self._lib.bf_workspace_bytes(C.byref(self._shape), a.n)
+        need = self._lib.bf_workspace_bytes(C.byref(self._shape), a.n) if self.wstream is not None else 0
         if getattr(self, "workspace", None) is None or self.workspace.numel() < need:
             self.workspace = torch.empty(need, device=self.device, dtype=torch.uint8)
-        a.workspace, a.workspace_bytes = self.workspace.data_ptr(), self.workspace.numel()
+        if need:
+            a.workspace, a.workspace_bytes = self.workspace.data_ptr(), self.workspace.numel()
         a.taps = C.pointer(taps) if taps is not None else None
         return a
+
+    def kernel_choice(self, n: int) -> str:
+        """Which kernel a call with ``n`` positions runs ("quad" or "board")."""
+        a = _Args()
+        a.n, a.shape, a.quant, a.kernel = n, self._shape, (1 if self.fp8 else 0), self.KERNELS[self.kernel]
+        a.wstream = a.fparams = 16 if self.wstream is not None else None        # only tested for NULL
+        a.board_wstream = a.board_fparams = 16 if self.board_wstream is not None else None
+        rc = self._lib.bf_kernel_choice(C.byref(a))
+        if rc < 0:
+            raise RuntimeError(f"bf_kernel_choice failed ({rc}): {self._lib.bf_last_error().decode()}")
+        return {1: "quad", 2: "board"}[rc]
 
     def _call(self, args: _Args) -> None:
         rc = self._lib.bf_model_forward(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream))

@@ -29,8 +29,10 @@
  *
  * Reduction orders fixed here ("lane order"): channels of a 32-wide tile are visited as
  *   ch(r, g) = 8 * (r / 4) + 4 * g + (r % 4),  r = 0..15, g = 0..1
- *   - row sums (LayerNorm mean / variance, softmax denominator): two partial sums, one
- *     per g, each accumulated sequentially over tiles then r; total = part[0] + part[1]
+ *   - row sums: two partial sums, one per g; total = part[0] + part[1].  The softmax
+ *     denominator accumulates each sequentially over r; LayerNorm mean / variance form each
+ *     from four group sums (a quarter of the tiles each, sequential over tiles then r)
+ *     added in group order, ((s0 + s1) + s2) + s3
  *   - dot products (QK^T, PV, heads): one fused-multiply-add chain over tiles, then r,
  *     then g, starting from +0
  *
@@ -182,23 +184,34 @@ static void layernorm_rows(const float* x, int d, const float* gamma, const floa
                            float eps, float* y) {
     for (int t = 0; t < T; t++) {
         const float* row = x + (size_t)t * d;
+        /* per lane half g: four group sums (a quarter of the tiles each, sequential over
+         * tiles then r) added in group order; then the two halves */
+        const int tq = d / 32 / 4;
         float part[2];
         for (int g = 0; g < 2; g++) {
-            float s = 0.0f;
-            for (int n = 0; n < d / 32; n++)
-                for (int r = 0; r < 16; r++) s = s + row[32 * n + ch(r, g)];
-            part[g] = s;
+            float sg[4];
+            for (int q = 0; q < 4; q++) {
+                float s = 0.0f;
+                for (int n = q * tq; n < (q + 1) * tq; n++)
+                    for (int r = 0; r < 16; r++) s = s + row[32 * n + ch(r, g)];
+                sg[q] = s;
+            }
+            part[g] = ((sg[0] + sg[1]) + sg[2]) + sg[3];
         }
         const float inv_d = 1.0f / (float)d; /* d is a power of two: exact */
         const float mean = (part[0] + part[1]) * inv_d;
         for (int g = 0; g < 2; g++) {
-            float s = 0.0f;
-            for (int n = 0; n < d / 32; n++)
-                for (int r = 0; r < 16; r++) {
-                    const float dv = row[32 * n + ch(r, g)] - mean;
-                    s = fmaf(dv, dv, s);
-                }
-            part[g] = s;
+            float sg[4];
+            for (int q = 0; q < 4; q++) {
+                float s = 0.0f;
+                for (int n = q * tq; n < (q + 1) * tq; n++)
+                    for (int r = 0; r < 16; r++) {
+                        const float dv = row[32 * n + ch(r, g)] - mean;
+                        s = fmaf(dv, dv, s);
+                    }
+                sg[q] = s;
+            }
+            part[g] = ((sg[0] + sg[1]) + sg[2]) + sg[3];
         }
         const float var = (part[0] + part[1]) * inv_d;
         const float rstd = 1.0f / sqrtf(var + eps);

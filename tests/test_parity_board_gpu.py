@@ -1,0 +1,171 @@
+"""Parity of the one-position-per-workgroup kernel, through the C-ABI.
+
+Same bar as tests/test_parity_gpu.py: operand bytes, int32 accumulators, residual stream, logits,
+value and masked argmax bit-identical to the C checker.  For the 256-wide network the kernel must
+also return exactly what the four-positions-per-workgroup kernel returns (the library picks
+between them by batch size, and a position's result may not depend on the batch it is in); for the
+512-wide, 16-head, 16-layer network (two 256-deep k-chunks per matmul of the width, eight for the
+second feed-forward matmul, summed in float64) it is the only kernel.
+"""
+import numpy as np
+import pytest
+import torch
+
+from brokefish_amd import encoder_impl, positions
+from brokefish_amd.net import BrokefishNet
+from oracle import c_oracle
+
+pytestmark = pytest.mark.gpu
+
+TAPS = ["embed", "qa_qkv", "acc_qkv", "qa_out", "acc_out", "qa_ff1", "acc_ff1", "qa_ff2", "acc_ff2", "resid", "normed"]
+
+
+def _make(d, heads, layers, nv=1, seed=0):
+    torch.manual_seed(seed)
+    net = BrokefishNet(d_model=d, n_heads=heads, d_ff=4 * d, n_layers=layers, n_value=nv).eval()
+    net.randomise_layers_(seed=seed + 3)
+    sd = {k: v.detach() for k, v in net.state_dict().items()}
+    return net, sd
+
+
+@pytest.fixture(scope="module")
+def base():
+    net, sd = _make(256, 8, 8)
+    return (net, sd, encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="board"),
+            encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="quad"), c_oracle.COracle(sd))
+
+
+@pytest.fixture(scope="module")
+def stress():
+    net, sd = _make(512, 16, 16)
+    return net, sd, encoder_impl("hip")(net, int8=True, out_dtype=torch.float32), c_oracle.COracle(sd)
+
+
+def _dev(*ts):
+    return [t.cuda() for t in ts]
+
+
+def _bits_equal(a: torch.Tensor, b: np.ndarray) -> bool:
+    a = a.cpu().numpy()
+    if a.dtype == np.uint8:
+        b = b.view(np.uint8)
+    return a.shape == b.shape and bool((a.view(np.int32 if a.dtype == np.float32 else a.dtype)
+                                        == b.view(np.int32 if b.dtype == np.float32 else b.dtype)).all())
+
+
+def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base):
+    net, sd, board, quad, co = base
+    b, c, r, m = positions.random_positions(48, plies=120, seed=11, stamp_queen=True)
+    got = board.forward_taps(*_dev(b, c, r), mask=m.cuda())
+    want = co.forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy(), taps=True)
+    for k in TAPS + ["policy", "promo", "value", "best"]:
+        assert _bits_equal(got[k], want[k]), k
+
+
+@pytest.mark.parametrize("nv", [1, 3])
+def test_the_two_kernels_return_the_same_bits(base, nv):
+    if nv == 1:
+        net, sd, board, quad, co = base
+    else:
+        net, sd = _make(256, 8, 8, nv=3, seed=5)
+        board = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="board")
+        quad = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="quad")
+    b, c, r, m = positions.random_positions(301, plies=120, seed=21)           # odd on purpose
+    bd, cd, rd, md = _dev(b, c, r, m)
+    pq, qq, vq = [t.clone() for t in quad.forward_full(bd, cd, rd, md)]
+    bestq = quad.best_move.clone()
+    pb, qb, vb = board.forward_full(bd, cd, rd, md)
+    assert torch.equal(pb, pq) and torch.equal(qb, qq) and torch.equal(vb, vq) and torch.equal(board.best_move, bestq)
+    raw_q = quad.forward_full(bd, cd, rd)[0].clone()
+    assert torch.equal(board.forward_full(bd, cd, rd)[0], raw_q) and torch.isfinite(raw_q).all()
+    one = board.forward_full(bd[7:8], cd[7:8], rd[7:8])[0]
+    assert torch.equal(one, raw_q[7:8])
+    half_b = encoder_impl("hip")(net, int8=True, kernel="board").forward_full(bd, cd, rd)[0]
+    assert half_b.dtype is torch.float16 and torch.equal(half_b, raw_q.half())
+    # teacher-forced single layers and the heads alone agree as well
+    x = torch.randn(301, 32, 256, generator=torch.Generator().manual_seed(3)).cuda()
+    for l0, l1 in ((2, 3), (5, 8), (8, 8)):
+        tb = board.forward_taps(bd, cd, rd, x_in=x, layer_begin=l0, layer_end=l1, want=["resid", "acc_ff2", "normed"])
+        tq = quad.forward_taps(bd, cd, rd, x_in=x, layer_begin=l0, layer_end=l1, want=["resid", "acc_ff2", "normed"])
+        for k in ("resid", "acc_ff2", "normed", "policy", "value"):
+            assert torch.equal(tb[k], tq[k]), (l0, l1, k)
+
+
+def test_automatic_choice_switches_kernel_by_batch_size_without_changing_results(base):
+    net, sd, board, quad, co = base
+    auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
+    cut = int(auto._lib.bf_board_max_n())
+    assert auto.kernel_choice(1) == "board" and auto.kernel_choice(cut) == "board"
+    assert auto.kernel_choice(cut + 1) == "quad" and auto.kernel_choice(4096) == "quad"
+    assert "by batch size" in auto.label
+    b, c, r, m = positions.random_positions(cut + 4, plies=120, seed=22)
+    bd, cd, rd, md = _dev(b, c, r, m)
+    big = [t.clone() for t in auto.forward_masked(bd, cd, rd, md)]                        # quad
+    small = auto.forward_masked(bd[:cut], cd[:cut], rd[:cut], md[:cut])                  # board
+    for x, y in zip(big, small):
+        assert torch.equal(x[:cut], y)
+    fp8 = encoder_impl("hip")(net, fp8=True)
+    assert fp8.kernel_choice(1) == "quad"
+    with pytest.raises(NotImplementedError):
+        encoder_impl("hip")(net, fp8=True, kernel="board")
+
+
+def test_stress_network_bit_exact_against_the_c_checker_with_every_tap(stress):
+    net, sd, model, co = stress
+    assert model.kernel_choice(16384) == "board" and model.wstream is None
+    b, c, r, m = positions.random_positions(12, plies=120, seed=31, stamp_queen=True)
+    got = model.forward_taps(*_dev(b, c, r), mask=m.cuda())
+    want = co.forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy(), taps=True)
+    for k in TAPS + ["policy", "promo", "value", "best"]:
+        assert _bits_equal(got[k], want[k]), k
+    assert got["acc_qkv"].shape == (12, 16, 2, 32, 1536) and got["acc_ff2"].shape == (12, 16, 8, 32, 512)
+    # the accumulators are the exact integer products of the kernel's own operand bytes, per k-chunk
+    q, _ = co.qweight("ff2", 9)
+    a = got["qa_ff2"][:, 9].cpu().numpy().astype(np.int64)                     # [n,32,2048] unsigned
+    acc = np.stack([a[..., 256 * k:256 * k + 256] @ q[:, 256 * k:256 * k + 256].astype(np.int64).T for k in range(8)], 1)
+    assert (acc == got["acc_ff2"][:, 9].cpu().numpy()).all()
+    q, _ = co.qweight("qkv", 15)
+    a = got["qa_qkv"][:, 15].cpu().numpy().astype(np.int64)
+    acc = np.stack([a[..., 256 * k:256 * k + 256] @ q[:, 256 * k:256 * k + 256].astype(np.int64).T for k in range(2)], 1)
+    assert (acc == got["acc_qkv"][:, 15].cpu().numpy()).all()
+    # production launch, fp16 contract, teacher forcing of a layer range and of the heads alone
+    bd, cd, rd, md = _dev(b, c, r, m)
+    p, q2, v = model.forward_full(bd, cd, rd, md)
+    assert torch.equal(p, got["policy"]) and torch.equal(q2, got["promo"]) and torch.equal(v, got["value"])
+    assert torch.equal(model.best_move, got["best"])
+    half = encoder_impl("hip")(net, int8=True).forward_full(bd, cd, rd, md)[0]
+    assert half.dtype is torch.float16 and torch.equal(half, p.half())
+    x_in = torch.from_numpy(want["resid"][:, 10]).cuda()
+    tail = model.forward_taps(bd, cd, rd, mask=md, x_in=x_in, layer_begin=11, layer_end=16, want=["resid"])
+    assert _bits_equal(tail["resid"][:, -1], want["resid"][:, 15]) and torch.equal(tail["policy"], got["policy"])
+    mid = model.forward_taps(bd, cd, rd, x_in=x_in, layer_begin=11, layer_end=12, want=["resid"])
+    assert _bits_equal(mid["resid"][:, 0], want["resid"][:, 11])
+    heads = model.forward_taps(bd, cd, rd, mask=md, x_in=torch.from_numpy(want["resid"][:, 15]).cuda(),
+                               layer_begin=16, layer_end=16, want=["normed"])
+    assert torch.equal(heads["policy"], got["policy"]) and torch.equal(heads["value"], got["value"])
+    with pytest.raises(NotImplementedError):
+        encoder_impl("hip")(net, fp8=True)
+    with pytest.raises(NotImplementedError):
+        encoder_impl("hip")(net, int8=True, kernel="quad")
+
+
+def test_stress_network_win_draw_loss_head_and_full_batch_properties():
+    # the configuration's batch size, 16384 positions: spot-check against the C checker,
+    # size-independent properties on everything
+    net, sd = _make(512, 16, 16, nv=3, seed=2)
+    model = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
+    co = c_oracle.COracle(sd)
+    n = 16384
+    b, c, r, m = positions.random_positions(n, plies=120, seed=0)
+    bd, cd, rd, md = _dev(b, c, r, m)
+    p, q, v, best = [t.clone() for t in model.forward_masked(bd, cd, rd, md)]
+    idx = np.arange(5, n, 2731)
+    want = co.forward(b.numpy()[idx], c.numpy()[idx], r.numpy()[idx], mask=m.numpy()[idx])
+    assert _bits_equal(p[idx], want["policy"]) and _bits_equal(q[idx], want["promo"])
+    assert _bits_equal(v[idx], want["value"]) and (best.cpu().numpy()[idx] == want["best"]).all()
+    part = model.forward_masked(bd[9000:9700], cd[9000:9700], rd[9000:9700], md[9000:9700])
+    assert torch.equal(part[0], p[9000:9700]) and torch.equal(part[3], best[9000:9700])
+    legal = ((md[..., None] >> torch.arange(64, device="cuda")) & 1).bool()
+    assert torch.isneginf(p[~legal]).all() and torch.isfinite(p[legal]).all() and (v.abs() <= 1).all()
+    has = legal.reshape(n, -1).any(1)
+    assert torch.gather(legal.reshape(n, -1)[has], 1, best[has].long()[:, None]).all()
