@@ -22,6 +22,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 OPS_PER_EVAL = 402_653_184            # 2 * 32 tokens * 8 layers * 12 * 256^2 int8 ops in the weight GEMMs
+OPS_PER_EVAL_STRESS = 3_221_225_472   # 2 * 32 tokens * 16 layers * 12 * 512^2 (the 512-wide, 16-layer network)
 PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s (dense fp8 MFMA: the same figure)
 # HBM bytes per launch of the default workload (batch 4096), from the FETCH_SIZE / WRITE_SIZE
 # counter runs summarised in profiles/eval_kernel_int8_batch4096.md (calibrated on a 1 GiB copy).
@@ -59,9 +60,14 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--batch", type=int, default=4096)
+    ap.add_argument("--batch", type=int, default=None, help="default 4096 (base) / 16384 (stress)")
     ap.add_argument("--quant", choices=("int8", "e4m3"), default="int8",
                     help="operand format of the weight matmuls; int8 is the headline metric, e4m3 the fp8 variant")
+    ap.add_argument("--shape", choices=("base", "stress"), default="base",
+                    help="base: 8 layers, width 256 (the headline metric); stress: 16 layers, width 512, "
+                         "16 heads, default batch 16384")
+    ap.add_argument("--kernel", choices=("auto", "quad", "board", "twin"), default="auto",
+                    help="four positions per workgroup; one position per workgroup with one (board) or two (twin) workgroups per compute unit; auto: by batch size")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=64)
     ap.add_argument("--sweep", action="store_true",
@@ -79,10 +85,16 @@ def main() -> int:
     from brokefish_amd import encoder_impl, positions
     from brokefish_amd.net import BrokefishNet
 
+    stress = a.shape == "stress"
+    if a.batch is None:
+        a.batch = 16384 if stress else 4096
+    ops_per_eval = OPS_PER_EVAL_STRESS if stress else OPS_PER_EVAL
     torch.manual_seed(0)
-    net = BrokefishNet().eval()                                  # seed-0 random init, reference init rules
+    # seed-0 random init, reference init rules
+    net = (BrokefishNet(d_model=512, n_heads=16, d_ff=2048, n_layers=16) if stress else BrokefishNet()).eval()
     fp8 = a.quant == "e4m3"
-    model = encoder_impl("hip")(net, fp8=True) if fp8 else encoder_impl("hip")(net, int8=True)   # fp16 logits: the search contract
+    # fp16 logits: the search contract
+    model = encoder_impl("hip")(net, fp8=True, kernel=a.kernel) if fp8 else encoder_impl("hip")(net, int8=True, kernel=a.kernel)
     b, c, r, m = positions.random_positions(a.batch, plies=120, seed=0)
     bd, cd, rd, md = b.cuda(), c.cuda(), r.cuda(), m.cuda()
 
@@ -104,19 +116,22 @@ def main() -> int:
     evals = a.batch * a.steps / dt
 
     kern_ms = model.time_kernel_ms(bd, cd, rd, md, warmup=3, iters=max(a.steps, 10))
-    achieved = OPS_PER_EVAL * a.batch / (kern_ms * 1e-3) / 1e12
+    achieved = ops_per_eval * a.batch / (kern_ms * 1e-3) / 1e12
     line = {
-        "metric": f"network evals/sec at batch 4096 {'fp8 e4m3' if fp8 else 'int8'} on 1 MI355X",
+        "metric": (f"network evals/sec at batch {a.batch} int8, 16-layer width-512 stress shape, on 1 MI355X" if stress
+                   else f"network evals/sec at batch 4096 {'fp8 e4m3' if fp8 else 'int8'} on 1 MI355X"),
         "value": evals, "unit": "evals/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8" if fp8 else "int8", "data": "synthetic",
-        "config": {"workload": f"configs[{4 if fp8 else 1}]: 8-layer d256 8-head FFN1024 {a.quant} evaluator, batch {a.batch}, "
+        "config": {"workload": (f"configs[4]: 16-layer d512 16-head FFN2048 int8 evaluator, batch {a.batch}, " if stress else
+                                f"configs[{3 if fp8 else 1}]: 8-layer d256 8-head FFN1024 {a.quant} evaluator, batch {a.batch}, ")
+                               + f"kernel {model.kernel_choice(a.batch)}, "
                                "seeded random playouts 0-120 plies, legal-move mask ANDed in-kernel, "
                                "fp16 logits out, seed-0 random-init weights"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
                      "frac": achieved / (PEAK_INT8_OPS / 1e12),
-                     "traffic": None if fp8 else MEASURED_TRAFFIC_BYTES.get(a.batch),
-                     "kernel_ms": kern_ms, "ops_per_launch": OPS_PER_EVAL * a.batch},
+                     "traffic": None if (fp8 or stress or model.kernel_choice(a.batch) != "quad") else MEASURED_TRAFFIC_BYTES.get(a.batch),
+                     "kernel_ms": kern_ms, "ops_per_launch": ops_per_eval * a.batch},
     }
     if a.sweep:
         # the batch-size sweep of the small-batch latency regime: same net, same generator
@@ -124,7 +139,8 @@ def main() -> int:
         for nb in (64, 256, 1024, 4096, 16384, 65536):
             sb, sc, sr, sm = (t.cuda() for t in positions.random_positions(nb, plies=120, seed=0))
             ms = model.time_kernel_ms(sb, sc, sr, sm, warmup=3, iters=20)
-            pts.append({"batch": nb, "ms_per_launch": ms, "evals_per_s": nb / ms * 1e3})
+            pts.append({"batch": nb, "ms_per_launch": ms, "evals_per_s": nb / ms * 1e3,
+                        "kernel": model.kernel_choice(nb)})
             del sb, sc, sr, sm
         line["sweep"] = pts
     if not a.no_cpu:

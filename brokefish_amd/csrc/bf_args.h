@@ -71,19 +71,21 @@ constexpr int G_SQ = 0, G_TS = 64 * D, G_CT = G_TS + 12 * D, G_CLOCK = G_CT + 4 
 
 // Layout of the one-position-per-workgroup kernel (bf_board.hip.h), for model width DM: wave w
 // owns tiles TW*w .. TW*w+TW-1 of the width.  Per layer a wave streams BPW weight blocks in its
-// own consumption order and reads PW_FLOATS side parameters (part A: attention phase, part B:
-// feed-forward phase); see include/brokefish_hip.h for the blob layouts.
+// own consumption order (the feed-forward block in STEPS of 512 hidden channels, of which a wave
+// computes four tiles) and reads PW_FLOATS side parameters (part A: attention phase, part B:
+// feed-forward phase).  A wave's stream is L * BPW layer blocks, HB head blocks and one block of
+// padding (the register prefetch runs one block ahead); see include/brokefish_hip.h.
 template <int DM>
 struct Layout {
     static constexpr int D = DM, F = 4 * DM, NT = DM / 32, TW = NT / 4, CW = 32 * TW, KC = DM / 256,
-                         KCF = F / 256, HALVES = F / 1024;
-    static constexpr int BPW = 3 * TW * KC + TW * KC + HALVES * (8 * KC + 4 * TW);
-    static constexpr int HB = NT / 2;              // head blocks per wave (8 fp32 fragments each)
-    static constexpr int SLOTS = DM == 256 ? 3 : 2;  // depth of a wave's private weight ring, in blocks
+                         KCF = F / 256, STEPS = F / 512;
+    static constexpr int BPW = 3 * TW * KC + TW * KC + STEPS * (4 * KC + 2 * TW);
+    static constexpr int HB = NT / 2;                // head blocks per wave (8 fp32 fragments each)
+    static constexpr int SLOTS = DM == 256 ? 3 : 2;  // depth of a wave's private LDS weight ring, in blocks
     static constexpr int A_LN1G = 0, A_LN1B = CW, A_BQ = 2 * CW, A_BK = 3 * CW, A_BV = 4 * CW, A_BOUT = 5 * CW,
                          A_SW = 6 * CW, A_FLOATS = 6 * CW + 16;
-    static constexpr int B_LN2G = 0, B_LN2B = CW, B_BFF1 = 2 * CW, B_BFF2 = 2 * CW + 256 * HALVES,
-                         B_WSUM = 3 * CW + 256 * HALVES, B_SW = B_WSUM + KCF * CW, B_FLOATS = B_SW + 32;
+    static constexpr int B_LN2G = 0, B_LN2B = CW, B_BFF1 = 2 * CW, B_BFF2 = 2 * CW + 128 * STEPS,
+                         B_WSUM = 3 * CW + 128 * STEPS, B_SW = B_WSUM + KCF * CW, B_FLOATS = B_SW + 32;
     static constexpr int PW_FLOATS = A_FLOATS + B_FLOATS;
     static constexpr int G_SQ = 0, G_TS = 64 * D, G_CT = G_TS + 12 * D, G_CLOCK = G_CT + 4 * D,
                          G_REP = G_CLOCK + 101 * D, G_NFG = G_REP + 3 * D, G_NFB = G_NFG + D,
@@ -125,5 +127,8 @@ hipError_t launch_board256(const KArgs& k, hipStream_t stream);
 hipError_t launch_board256_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_board512(const KArgs& k, hipStream_t stream);
 hipError_t launch_board512_taps(const KArgs& k, hipStream_t stream);
+// the same with two workgroups per compute unit (256-wide network)
+hipError_t launch_twin256(const KArgs& k, hipStream_t stream);
+hipError_t launch_twin256_taps(const KArgs& k, hipStream_t stream);
 
 }  // namespace bf

@@ -2,20 +2,31 @@
 //
 // Wavefront w owns a quarter of the channels of the residual stream (tiles TW*w .. TW*w+TW-1,
 // which are also its attention heads), a quarter of every matmul's output tiles, and streams
-// exactly the weight blocks of those tiles through a private LDS ring (no cross-wave
-// synchronisation for weights).  Quantised activations are exchanged through LDS as ready-made
-// MFMA B-operand fragments; row statistics (LayerNorm sums, quantiser maxima) are exchanged as
+// exactly the weight blocks of those tiles -- privately, so weights need no cross-wave
+// synchronisation.  Quantised activations are exchanged through LDS as ready-made MFMA
+// B-operand fragments; row statistics (LayerNorm sums, quantiser maxima) are exchanged as
 // per-lane partials and combined in wave order, which is the group order of the arithmetic
 // contract in bf_args.h -- so for the 256-wide network this kernel returns bit for bit what the
-// one-wavefront-per-position kernel returns.
+// one-wavefront-per-position kernel returns.  The feed-forward block runs in steps of 512 hidden
+// channels: each wave computes four hidden tiles per step, so a 256-wide quantiser chunk spans a
+// pair of waves and its maximum is exchanged; the float64 sums over the chunks stay in order.
 //
-// It serves two purposes: launches too small to fill the GPU with four positions per workgroup
-// (latency: four times the parallelism per position), and the 512-wide network, whose residual
-// stream does not fit one wavefront's registers.
+// Two forms, selected by TWIN, with identical results:
+//   TWIN = false  one workgroup per compute unit, 512 registers per wave.  Weight blocks stream
+//                 through a private LDS ring per wave (direct-to-LDS loads, SLOTS blocks deep),
+//                 attention is software-pipelined across heads.  Lowest latency per position
+//                 (launches of up to one position per compute unit) and the only form the
+//                 512-wide network fits.
+//   TWIN = true   two workgroups per compute unit: at most 80 KiB of LDS and 256 registers per
+//                 wave, so every SIMD holds two wavefronts of different positions and one's
+//                 waits (LDS round trips, barriers, MFMA results) are covered by the other's
+//                 work.  Weight fragments go from L2 straight to registers (half a block = four
+//                 fragments at a time, prefetched one block ahead through three register sets).
+//                 Highest throughput.
 //
-// LDS map (bytes): [ring: 4 waves x SLOTS x 8 KiB] [xch: 3 KiB] [hid: 32 KiB] [act: NT KiB]
-// [par: 4 waves x PW floats].  During the heads the normalised stream (NT*4 KiB, fp32) overlays
-// hid/act/par.
+// LDS map (bytes): [ring: 4 waves x SLOTS x 8 KiB, absent in the TWIN form] [xch: 3 KiB]
+// [hid: 16 KiB] [act: NT KiB] [par: 4 waves x PW floats].  During the heads the normalised stream
+// (NT*4 KiB, fp32) overlays hid/act/par.
 #pragma once
 
 #include "bf_device.hip.h"
@@ -25,17 +36,19 @@ namespace board {
 
 extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
-template <int DM>
+template <int DM, bool TWIN>
 struct Cfg : Layout<DM> {
     typedef Layout<DM> L;
-    static constexpr int XCH_OFF = 4 * L::SLOTS * BLOCK;
+    static constexpr int RING_BYTES = TWIN ? 0 : 4 * L::SLOTS * BLOCK;
+    static constexpr int XCH_OFF = RING_BYTES;
     static constexpr int HID_OFF = XCH_OFF + 3 * FRAG;
-    static constexpr int ACT_OFF = HID_OFF + 32 * FRAG;
+    static constexpr int ACT_OFF = HID_OFF + 16 * FRAG;
     static constexpr int PAR_OFF = ACT_OFF + L::NT * FRAG;
     static constexpr int LDS_BYTES = PAR_OFF + 4 * L::PW_FLOATS * 4;
-    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one compute unit");
+    static_assert(LDS_BYTES <= (TWIN ? 80 : 160) * 1024, "LDS budget: one or two workgroups per compute unit");
     static_assert(L::NT * 4 * FRAG <= LDS_BYTES - HID_OFF, "normalised stream overlay");
     static_assert(L::BPW % L::SLOTS == 0, "ring slot of a block must not depend on the layer");
+    static_assert((2 * L::BPW) % 3 == 0, "register set of a half-block must not depend on the layer");
 };
 
 // workgroup barrier that waits for this wave's LDS traffic only (outstanding direct-to-LDS
@@ -78,19 +91,20 @@ __device__ __forceinline__ float chunk_sum(const v16i (&acc)[KC], int i, const f
     }
 }
 
-template <int DM, bool TAPS>
-__global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
-    typedef Cfg<DM> C;
+template <int DM, bool TAPS, bool TWIN>
+__global__ __launch_bounds__(THREADS, TWIN ? 2 : 1) void board_kernel(const KArgs a) {
+    typedef Cfg<DM, TWIN> C;
     constexpr int D = C::D, F = C::F, NT = C::NT, TW = C::TW, CW = C::CW, KC = C::KC, KCF = C::KCF;
-    constexpr int HALVES = C::HALVES, BPW = C::BPW, HB = C::HB, SLOTS = C::SLOTS, WPC = 4 / KC;
-    constexpr int VM_AHEAD = TAPS ? 0 : (SLOTS - 1) * 8;   // weight loads that may stay in flight at a ring wait
+    constexpr int STEPS = C::STEPS, BPW = C::BPW, HB = C::HB, SLOTS = C::SLOTS, WPC = 4 / KC;
+    constexpr int HALF = BLOCK / 2;   // four fragments: the unit of the register prefetch (TWIN)
+    constexpr int VM_AHEAD = TAPS ? 0 : (SLOTS - 1) * 8;   // ring loads that may stay in flight at a ring wait
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t = lane & 31, g = lane >> 5;
     const int b = blockIdx.x;
     const int nl_run = a.l1 - a.l0;
 
-    uint8_t* const myring = lds + wave * (SLOTS * BLOCK);
+    uint8_t* const myring = lds + wave * (SLOTS * BLOCK);   // !TWIN
     float* const xch = reinterpret_cast<float*>(lds + C::XCH_OFF);
     uint8_t* const hid = lds + C::HID_OFF;
     uint8_t* const act = lds + C::ACT_OFF;
@@ -98,10 +112,19 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
     float* const pB = pA + C::A_FLOATS;
     // this wave's weight stream, from the first layer that runs; block `seq` in consumption order
     const uint8_t* const wsrc =
-        a.wstream + ((size_t)wave * ((size_t)a.n_layers * BPW + HB) + (size_t)a.l0 * BPW) * BLOCK + lane * 16;
+        a.wstream + ((size_t)wave * ((size_t)a.n_layers * BPW + HB + 1) + (size_t)a.l0 * BPW) * BLOCK + lane * 16;
     const float* const wpar = a.fparams + (size_t)wave * a.n_layers * C::PW_FLOATS;   // this wave's [layer][PW]
     const float* const gp = a.fparams + (size_t)4 * a.n_layers * C::PW_FLOATS;       // tables, final norm
 
+    // TWIN: half-block `hseq` of this wave's stream (consumption order) into register set `set`
+    v4i frt[3][4];
+    auto load_half = [&](int hseq, int set) {
+        const uint8_t* src = wsrc + (size_t)hseq * HALF;
+#pragma unroll
+        for (int s = 0; s < 4; s++) frt[set][s] = *reinterpret_cast<const v4i*>(src + s * FRAG);
+    };
+    // !TWIN: block `seq` into ring slot `slot`; a slot into the fragment registers
+    v4i fr[8];
     auto issue_block = [&](int seq, int slot) {
         const uint8_t* src = wsrc + (size_t)seq * BLOCK;
         uint8_t* dst = myring + slot * BLOCK;
@@ -110,7 +133,6 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + s * FRAG),
                                              (__attribute__((address_space(3))) void*)(dst + s * FRAG), 16, 0, 0);
     };
-    v4i fr[8];
     auto read_slot = [&](int slot) {
 #pragma unroll
         for (int s = 0; s < 8; s++) fr[s] = *reinterpret_cast<const v4i*>(&myring[slot * BLOCK + s * FRAG + lane * 16]);
@@ -193,8 +215,13 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
     };
 
     // ---- start the weight stream and the first layer's parameters ------------------------------
+    if constexpr (TWIN) {
+        load_half(0, 0);
+        load_half(1, 1);
+    } else {
 #pragma unroll
-    for (int j = 0; j < SLOTS; j++) issue_block(j, j);
+        for (int j = 0; j < SLOTS; j++) issue_block(j, j);
+    }
     if (nl_run > 0) {
         dma(wpar + (size_t)a.l0 * C::PW_FLOATS, pA, C::A_FLOATS, lane);
         dma(wpar + (size_t)a.l0 * C::PW_FLOATS + C::A_FLOATS, pB, C::B_FLOATS, lane);
@@ -252,24 +279,42 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
             for (int r = 0; r < 16; r++)
                 a.taps.embed[((size_t)b * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = x[i][r];
 
-    // everything issued so far has landed: parameters, and the first SLOTS weight blocks
-    wait_vm<0>();
-    read_slot(0);
+    wait_vm<0>();   // the parameters (and the first ring slots) have landed
+    if constexpr (!TWIN) read_slot(0);
 
     for (int l = a.l0; l < a.l1; l++) {
         const int li = l - a.l0;
         const size_t bl = (size_t)b * nl_run + li;   // tap row
         const int lnext = l + 1 < a.l1 ? l + 1 : l;  // after the last layer the same slice is fetched again
-        // Multiply by the block in `fr` (index k of this wave's layer), with the ring kept full:
-        // the slot `fr` came from is refilled SLOTS blocks ahead, then block k+1 is read.
-#define BF_WMM(SWAP, k, actp)                                                              \
-    ([&]() -> v16i {                                                                       \
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                 \
-        issue_block(li * BPW + (k) + SLOTS, (k) % SLOTS);                                  \
-        const v16i r_ = mfma8<SWAP, false>(fr, *reinterpret_cast<const v4i(*)[8]>(actp));  \
-        wait_vm<VM_AHEAD>();                                                               \
-        read_slot(((k) + 1) % SLOTS);                                                      \
-        return r_;                                                                         \
+        // Multiply by block k of this wave's layer.
+        // TWIN: its two halves sit in register sets 2k % 3 and (2k + 1) % 3; each half's set is
+        // refilled with the half three positions on once consumed.
+        // !TWIN: the block is in `fr`; the ring slot it came from is refilled SLOTS blocks ahead,
+        // then block k+1 is read from its slot.
+        const int hbase = li * 2 * BPW;
+#define BF_WMM(SWAP, k, actp)                                                                        \
+    ([&]() -> v16i {                                                                                 \
+        const v4i* act_ = (actp);                                                                    \
+        v16i r_ = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};                                  \
+        if constexpr (TWIN) {                                                                        \
+            load_half(hbase + 2 * (k) + 2, (2 * (k) + 2) % 3);                                       \
+            _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
+                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[s_], frt[(2 * (k)) % 3][s_], r_, 0, 0, 0)  \
+                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(frt[(2 * (k)) % 3][s_], act_[s_], r_, 0, 0, 0); \
+            load_half(hbase + 2 * (k) + 3, (2 * (k) + 3) % 3);                                       \
+            _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
+                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[4 + s_], frt[(2 * (k) + 1) % 3][s_], r_, 0, 0, 0)  \
+                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(frt[(2 * (k) + 1) % 3][s_], act_[4 + s_], r_, 0, 0, 0); \
+        } else {                                                                                     \
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                       \
+            issue_block(li * BPW + (k) + SLOTS, (k) % SLOTS);                                        \
+            _Pragma("unroll") for (int s_ = 0; s_ < 8; s_++)                                         \
+                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[s_], fr[s_], r_, 0, 0, 0)     \
+                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[s_], act_[s_], r_, 0, 0, 0);    \
+            wait_vm<VM_AHEAD>();                                                                     \
+            read_slot(((k) + 1) % SLOTS);                                                            \
+        }                                                                                            \
+        return r_;                                                                                   \
     }())
 
         // ---- LayerNorm 1, quantise, exchange ----------------------------------------------------------
@@ -286,17 +331,21 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; r++) sa_tok[c][r] = __shfl(sa[c], ch(r, g));
 
-        // ---- attention over this wave's heads, software-pipelined as in the other kernel ----------------
+        // ---- attention over this wave's heads ----------------------------------------------------------
+        // !TWIN: software-pipelined -- the three weight GEMMs of head i+1 are issued right after the
+        // score MFMAs of head i, so the matrix pipe works through them under head i's softmax.
         float o[TW][16];
         v16i accq[KC], acck[KC], accv[KC];
 #pragma unroll
-        for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, c, &xq[8 * c]);
-#pragma unroll
-        for (int c = 0; c < KC; c++) acck[c] = BF_WMM(false, KC + c, &xq[8 * c]);
-#pragma unroll
-        for (int c = 0; c < KC; c++) accv[c] = BF_WMM(true, 2 * KC + c, &xq[8 * c]);
-#pragma unroll
         for (int i = 0; i < TW; i++) {
+            if (TWIN || i == 0) {
+#pragma unroll
+                for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * i + c, &xq[8 * c]);
+#pragma unroll
+                for (int c = 0; c < KC; c++) acck[c] = BF_WMM(false, 3 * KC * i + KC + c, &xq[8 * c]);
+#pragma unroll
+                for (int c = 0; c < KC; c++) accv[c] = BF_WMM(true, 3 * KC * i + 2 * KC + c, &xq[8 * c]);
+            }
             const int h = TW * wave + i;
             float qf[16], kf[16], vf[16];
             {
@@ -334,7 +383,7 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
             v16f sc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
             for (int r = 0; r < 16; r++) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[r], qf[r], sc, 0, 0, 0);
-            if (i + 1 < TW) {
+            if (!TWIN && i + 1 < TW) {
 #pragma unroll
                 for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * (i + 1) + c, &xq[8 * c]);
 #pragma unroll
@@ -410,23 +459,24 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
         double o64[TW][16];
         constexpr int KF = 3 * KC * TW + KC * TW;   // first feed-forward block of the layer
 #pragma unroll
-        for (int hh = 0; hh < HALVES; hh++) {
-            constexpr int HBLK = 8 * KC + 4 * TW;   // blocks of one half
-            const int k1 = KF + hh * HBLK;          // first matmul: 8 hidden tiles of this wave = one 256-wide chunk
+        for (int st = 0; st < STEPS; st++) {
+            constexpr int SBLK = 4 * KC + 2 * TW;   // blocks of one step
+            const int k1 = KF + st * SBLK;          // first matmul: four hidden tiles of this wave (half a 256-wide chunk)
+            float sh[2];                            // scales of the step's two chunks
             {
-                float hf[8][16];
+                float hf[4][16];
                 float am = 0.0f;
                 v16i acc2[2][KC];
 #pragma unroll
                 for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + c, &xq[8 * c]);
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    if (i + 1 < 8)
+                for (int i = 0; i < 4; i++) {
+                    if (i + 1 < 4)
 #pragma unroll
                         for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, k1 + KC * (i + 1) + c, &xq[8 * c]);
                     v4f b1[4];
-                    load_tile16(pB + C::B_BFF1 + 256 * hh + 32 * i, g, b1);
-                    const float sw = pB[C::B_SW + 8 * hh + i];
+                    load_tile16(pB + C::B_BFF1 + 128 * st + 32 * i, g, b1);
+                    const float sw = pB[C::B_SW + 4 * st + i];
 #pragma unroll
                     for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -441,42 +491,49 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
                         for (int c = 0; c < KC; c++)
 #pragma unroll
                             for (int r = 0; r < 16; r++)
-                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 1024 * hh + 256 * wave + 32 * i + ch(r, g)] = acc2[i & 1][c][r];
+                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * wave + 32 * i + ch(r, g)] = acc2[i & 1][c][r];
                 }
-                // unsigned quantiser over this wave's chunk; bytes stored as q - 128 for the signed MFMA
-                am = __builtin_fmaxf(am, partner(am, g));
-                const float s8 = am > 0.0f ? am / 255.0f : 1.0f;
-                const float inv = 1.0f / s8;
-                xch[2 * 256 + wave * 64 + lane] = s8;   // slot 2: next written after the following layer's LayerNorm barriers
+                // unsigned quantiser over the 256-wide chunk this wave shares with its neighbour (waves
+                // 0,1: first chunk of the step; 2,3: second); bytes stored as q - 128 for the signed MFMA
+                xch[2 * 256 + wave * 64 + lane] = am;
+                lds_barrier();
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
+                for (int c = 0; c < 2; c++) {
+                    float m = __builtin_fmaxf(xch[2 * 256 + (2 * c) * 64 + lane], xch[2 * 256 + (2 * c + 1) * 64 + lane]);
+                    m = __builtin_fmaxf(m, partner(m, g));
+                    sh[c] = m > 0.0f ? m / 255.0f : 1.0f;
+                }
+                const float s8 = wave < 2 ? sh[0] : sh[1];
+                const float inv = 1.0f / s8;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
                     v4i w;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const unsigned u = quant4<false>(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
                         if (TAPS && a.taps.qa_ff2)
-                            *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 1024 * hh + 256 * wave + 32 * i + 8 * j + 4 * g) = u;
+                            *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 512 * st + 128 * wave + 32 * i + 8 * j + 4 * g) = u;
                         w[j] = (int)(u ^ 0x80808080u);
                     }
-                    *reinterpret_cast<v4i*>(hid + (8 * wave + i) * FRAG + lane * 16) = w;
+                    *reinterpret_cast<v4i*>(hid + (4 * wave + i) * FRAG + lane * 16) = w;
                 }
             }
             lds_barrier();
             // second matmul, chunk-major: one chunk of the hidden row (eight fragments) serves this
             // wave's TW output tiles; the float64 sums over the chunks stay in chunk order
-            const int k2 = k1 + 8 * KC;
+            const int k2 = k1 + 4 * KC;
             v16i acc2[2];
             v4i hqc[8];
 #pragma unroll
             for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + s * FRAG + lane * 16);
             acc2[0] = BF_WMM(false, k2, &hqc[0]);
 #pragma unroll
-            for (int idx = 0; idx < 4 * TW; idx++) {
+            for (int idx = 0; idx < 2 * TW; idx++) {
                 const int c = idx / TW, i = idx % TW;
-                const double sc = (double)xch[2 * 256 + c * 64 + lane];
+                const double sc = (double)sh[c];
                 v4i ws[4];
-                load_tile16i(pB + C::B_WSUM + (4 * hh + c) * CW + 32 * i, g, ws);
-                if (idx + 1 < 4 * TW) {
+                load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * i, g, ws);
+                if (idx + 1 < 2 * TW) {
                     if ((idx + 1) % TW == 0)
 #pragma unroll
                         for (int s = 0; s < 8; s++)
@@ -489,22 +546,20 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
 #pragma unroll
                     for (int k = 0; k < 4; k++) {
                         const int full = acc[4 * j + k] + ws[j][k];
-                        o64[i][4 * j + k] = (hh == 0 && c == 0) ? (double)full * sc
+                        o64[i][4 * j + k] = (st == 0 && c == 0) ? (double)full * sc
                                                                 : __builtin_fma((double)full, sc, o64[i][4 * j + k]);
                         if (TAPS && a.taps.acc_ff2)
-                            a.taps.acc_ff2[((bl * KCF + 4 * hh + c) * T + t) * D + 32 * (TW * wave + i) + 8 * j + 4 * g + k] = full;
+                            a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * wave + i) + 8 * j + 4 * g + k] = full;
                     }
 #pragma unroll
                 for (int r = 0; r < 16; r++) pin(o64[i][r]);
             }
-            // the next half overwrites the hidden buffer and the scale slots
-            if (hh + 1 < HALVES) lds_barrier();
         }
 #pragma unroll
         for (int i = 0; i < TW; i++) {
             v4f b2[4];
             load_tile16(pB + C::B_BFF2 + 32 * i, g, b2);
-            const float sw = pB[C::B_SW + 8 * HALVES + i];
+            const float sw = pB[C::B_SW + 16 + i];
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -523,16 +578,21 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
     }
 
     // ---- final norm and heads --------------------------------------------------------------------------
-    // `fr` holds the first head block unless a layer range that stops early left the blocks of the
-    // next layer in the ring: then restart the stream at the head blocks.
+    // The first head block is in the fragment registers unless a layer range that stops early left
+    // the blocks of the next layer there: then restart the stream at the head blocks.
     const int hseq0 = (a.n_layers - a.l0) * BPW;
     wait_vm<0>();   // also: no parameter copy is still landing where the normalised stream goes
     if (a.l1 != a.n_layers) {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if constexpr (TWIN) {
+            load_half(2 * hseq0, 0);
+            load_half(2 * hseq0 + 1, 1);
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-        for (int j = 0; j < SLOTS; j++) issue_block(hseq0 + j, j);
-        wait_vm<0>();
-        read_slot(0);
+            for (int j = 0; j < SLOTS; j++) issue_block(hseq0 + j, j);
+            wait_vm<0>();
+            read_slot(0);
+        }
     }
     float hn[TW][16];
     layernorm(x, gp + C::G_NFG + CW * wave, gp + C::G_NFB + CW * wave, hn);
@@ -555,20 +615,34 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
     // wave m multiplies head tile m (rows 32m..32m+31 of [policy; promo; value; 0]) over the whole
     // width, one fused-multiply-add chain in (tile, quad, element) order; wave 3's tile is zero
     v16f head = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (TWIN) {
 #pragma unroll
-    for (int hb = 0; hb < HB; hb++) {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (hb + SLOTS < HB) issue_block(hseq0 + hb + SLOTS, hb % SLOTS);
+        for (int hi = 0; hi < 2 * HB; hi++) {          // half-block = the four fragments (n = hi, q = 0..3)
+            load_half(2 * hseq0 + hi + 2, (hi + 2) % 3);   // the stream is padded by one block
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            const v4f w = __builtin_bit_cast(v4f, fr[s]);
-            const v4f hv = *reinterpret_cast<const v4f*>(hnb + ((hb * 8 + s) * 64 + lane) * 4);
+            for (int s = 0; s < 4; s++) {
+                const v4f w = __builtin_bit_cast(v4f, frt[hi % 3][s]);
+                const v4f hv = *reinterpret_cast<const v4f*>(hnb + ((hi * 4 + s) * 64 + lane) * 4);
 #pragma unroll
-            for (int k = 0; k < 4; k++) head = __builtin_amdgcn_mfma_f32_32x32x2f32(w[k], hv[k], head, 0, 0, 0);
+                for (int k = 0; k < 4; k++) head = __builtin_amdgcn_mfma_f32_32x32x2f32(w[k], hv[k], head, 0, 0, 0);
+            }
         }
-        if (hb + 1 < HB) {
-            wait_vm<0>();
-            read_slot((hb + 1) % SLOTS);
+    } else {
+#pragma unroll
+        for (int hb = 0; hb < HB; hb++) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (hb + SLOTS < HB) issue_block(hseq0 + hb + SLOTS, hb % SLOTS);
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                const v4f w = __builtin_bit_cast(v4f, fr[s]);
+                const v4f hv = *reinterpret_cast<const v4f*>(hnb + ((hb * 8 + s) * 64 + lane) * 4);
+#pragma unroll
+                for (int k = 0; k < 4; k++) head = __builtin_amdgcn_mfma_f32_32x32x2f32(w[k], hv[k], head, 0, 0, 0);
+            }
+            if (hb + 1 < HB) {
+                wait_vm<0>();
+                read_slot((hb + 1) % SLOTS);
+            }
         }
     }
 
@@ -649,17 +723,18 @@ __global__ __launch_bounds__(THREADS, 1) void board_kernel(const KArgs a) {
     }
 }
 
-template <int DM, bool TAPS>
+template <int DM, bool TAPS, bool TWIN>
 hipError_t launch_board(const KArgs& k, hipStream_t stream) {
     // more than 64 KiB of dynamic LDS has to be requested once per kernel (per thread: cheap)
     static thread_local bool lds_set = false;
+    constexpr int lds_bytes = Cfg<DM, TWIN>::LDS_BYTES;
     if (!lds_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&board_kernel<DM, TAPS>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, Cfg<DM>::LDS_BYTES);
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&board_kernel<DM, TAPS, TWIN>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess) return e;
         lds_set = true;
     }
-    hipLaunchKernelGGL((board_kernel<DM, TAPS>), dim3(k.n), dim3(THREADS), Cfg<DM>::LDS_BYTES, stream, k);
+    hipLaunchKernelGGL((board_kernel<DM, TAPS, TWIN>), dim3(k.n), dim3(THREADS), lds_bytes, stream, k);
     return hipGetLastError();
 }
 

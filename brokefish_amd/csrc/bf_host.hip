@@ -27,14 +27,15 @@ static bool shape512(const bf_shape* s) {
 
 static bool board_shape_ok(const bf_shape* s) { return shape_ok(s) || shape512(s); }
 
-// AUTO prefers one position per workgroup up to this many positions (256-wide network): below
-// it the four-per-workgroup launch leaves most compute units idle.
-static const int64_t kBoardMaxN = 768;
+// AUTO runs one workgroup per compute unit (lowest latency per position) up to this many
+// positions, which is one per compute unit of an MI355X; above it, two workgroups per compute
+// unit (highest throughput).
+static const int64_t kBoardMaxN = 256;
 
 template <int DM>
 static size_t board_wstream_bytes(int n_layers) {
     typedef bf::Layout<DM> L;
-    return (size_t)4 * ((size_t)n_layers * L::BPW + L::HB) * bf::BLOCK;
+    return (size_t)4 * ((size_t)n_layers * L::BPW + L::HB + 1) * bf::BLOCK;
 }
 template <int DM>
 static size_t board_fparams_floats(int n_layers) {
@@ -105,14 +106,18 @@ static int choose_kernel(const bf_eval_args* a) {
     case BF_KERNEL_BOARD:
         if (!board_can) return fail(BF_ERR_UNSUPPORTED, "the one-position-per-workgroup kernel needs board_wstream/board_fparams and the int8 format");
         return BF_KERNEL_BOARD;
+    case BF_KERNEL_TWIN:
+        if (!board_can || !shape_ok(&a->shape))
+            return fail(BF_ERR_UNSUPPORTED, "the two-workgroups-per-compute-unit kernel needs the 256-wide network, board_wstream/board_fparams and the int8 format");
+        return BF_KERNEL_TWIN;
     case BF_KERNEL_AUTO:
-        if (board_can && (!quad_can || a->n <= kBoardMaxN)) return BF_KERNEL_BOARD;
+        if (board_can) return (shape_ok(&a->shape) && a->n > kBoardMaxN) ? BF_KERNEL_TWIN : BF_KERNEL_BOARD;
         if (quad_can) return BF_KERNEL_QUAD;
         return fail(BF_ERR_ARGUMENT, shape512(&a->shape)
                         ? "the 512-wide network runs on the one-position-per-workgroup kernel: int8, board_wstream/board_fparams required"
                         : "wstream/fparams must not be NULL");
     default:
-        return fail(BF_ERR_ARGUMENT, "kernel must be BF_KERNEL_AUTO, BF_KERNEL_QUAD or BF_KERNEL_BOARD");
+        return fail(BF_ERR_ARGUMENT, "kernel must be BF_KERNEL_AUTO, BF_KERNEL_QUAD, BF_KERNEL_BOARD or BF_KERNEL_TWIN");
     }
 }
 
@@ -121,7 +126,7 @@ extern "C" int bf_kernel_choice(const bf_eval_args* args) { return choose_kernel
 static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     *kind = choose_kernel(a);
     if (*kind < 0) return *kind;
-    const bool board = *kind == BF_KERNEL_BOARD;
+    const bool board = *kind == BF_KERNEL_BOARD || *kind == BF_KERNEL_TWIN;
     if (a->n < 1 || a->n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
     if (!a->boards || !a->control || !a->rep) return fail(BF_ERR_ARGUMENT, "boards/control/rep must not be NULL");
     if (!a->policy || !a->promo || !a->value) return fail(BF_ERR_ARGUMENT, "policy/promo/value must not be NULL");
@@ -158,7 +163,10 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
 static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream_t stream) {
     const int grid = (k.n + bf::WAVES - 1) / bf::WAVES;
     hipError_t e;
-    if (kind == BF_KERNEL_BOARD) {
+    if (kind == BF_KERNEL_TWIN) {
+        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
+        e = a->taps ? bf::launch_twin256_taps(k, stream) : bf::launch_twin256(k, stream);
+    } else if (kind == BF_KERNEL_BOARD) {
         if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
         if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_board512_taps(k, stream) : bf::launch_board512(k, stream);

@@ -2,5 +2,5 @@
 #include "bf_board.hip.h"
 
 namespace bf {
-hipError_t launch_board256_taps(const KArgs& k, hipStream_t stream) { return board::launch_board<256, true>(k, stream); }
+hipError_t launch_board256_taps(const KArgs& k, hipStream_t stream) { return board::launch_board<256, true, false>(k, stream); }
 }  // namespace bf

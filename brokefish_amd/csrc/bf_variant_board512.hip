@@ -2,5 +2,5 @@
 #include "bf_board.hip.h"
 
 namespace bf {
-hipError_t launch_board512(const KArgs& k, hipStream_t stream) { return board::launch_board<512, false>(k, stream); }
+hipError_t launch_board512(const KArgs& k, hipStream_t stream) { return board::launch_board<512, false, false>(k, stream); }
 }  // namespace bf

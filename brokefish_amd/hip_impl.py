@@ -246,7 +246,7 @@ def pack_network_board(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: in
     of the one-position-per-workgroup kernel (layout at the end of include/brokefish_hip.h).
     Wave w owns tiles tw*w .. tw*w+tw-1 of the width; each wave gets its own weight stream and
     its own slice of the side parameters."""
-    nt, tw, kc, kcf, halves = d // 32, d // 128, d // 256, f // 256, f // 1024
+    nt, tw, kc, kcf = d // 32, d // 128, d // 256, f // 256
     cw = 32 * tw
     get = lambda k: sd[k].detach().float().cpu()
     quant = []
@@ -272,11 +272,11 @@ def pack_network_board(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: in
             for n in tiles:
                 for c in range(kc):
                     stream.append(pack_int8_block(q_out, n, 256 * c))
-            for hh in range(halves):
-                for i in range(8):
+            for st in range(f // 512):     # feed-forward in steps of 512 hidden channels, four tiles per wave
+                for i in range(4):
                     for c in range(kc):
-                        stream.append(pack_int8_block(q_ff1, 32 * hh + 8 * w + i, 256 * c))
-                for c in range(4 * hh, 4 * hh + 4):
+                        stream.append(pack_int8_block(q_ff1, 16 * st + 4 * w + i, 256 * c))
+                for c in range(2 * st, 2 * st + 2):
                     for n in tiles:
                         stream.append(pack_int8_block(q_ff2, n, 256 * c))
             b_qkv = get(p + "self_attn.in_proj_bias").numpy()
@@ -289,19 +289,20 @@ def pack_network_board(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: in
             part_a = [get(p + "norm1.weight").numpy()[own], get(p + "norm1.bias").numpy()[own],
                       b_qkv[:d][own], b_qkv[d:2 * d][own], b_qkv[2 * d:][own],
                       get(p + "self_attn.out_proj.bias").numpy()[own], sw_a]
-            hidden = np.concatenate([np.arange(1024 * hh + 256 * w, 1024 * hh + 256 * w + 256) for hh in range(halves)])
+            hidden = np.concatenate([np.arange(512 * st + 128 * w, 512 * st + 128 * w + 128) for st in range(f // 512)])
             wsum = (128 * q_ff2.astype(np.int32).reshape(d, kcf, 256).sum(axis=2)).T[:, own]   # [kcf, cw]
             sw_b = np.zeros(32, np.float32)
-            for hh in range(halves):
-                for i in range(8):
-                    sw_b[8 * hh + i] = s_ff1[(1024 * hh + 256 * w + 32 * i) // BLOCK_N]
+            for st in range(f // 512):
+                for i in range(4):
+                    sw_b[4 * st + i] = s_ff1[(512 * st + 128 * w + 32 * i) // BLOCK_N]
             for i, n in enumerate(tiles):
-                sw_b[8 * halves + i] = s_ff2[(32 * n) // BLOCK_N]
+                sw_b[16 + i] = s_ff2[(32 * n) // BLOCK_N]
             part_b = [get(p + "norm2.weight").numpy()[own], get(p + "norm2.bias").numpy()[own],
                       get(p + "linear1.bias").numpy()[hidden], get(p + "linear2.bias").numpy()[own],
                       np.ascontiguousarray(wsum, dtype=np.int32).view(np.float32).reshape(-1), sw_b]
             fl += part_a + part_b
         stream.append(pack_head_tile(head, w).view(np.uint8))
+        stream.append(np.zeros(8192, np.uint8))     # the weight prefetch runs one block past the end
     for name in ("emb_square", "emb_type_special", "emb_color_turn", "emb_clock", "emb_rep"):
         fl.append(get(name + ".weight").numpy())
     fl += [get("norm_f.weight").numpy(), get("norm_f.bias").numpy()]
@@ -319,7 +320,7 @@ class FusedEncoder:
 
     D, DFF, T, H = 256, 1024, 32, 8
     SHAPES = ((256, 1024, 8), (512, 2048, 16))     # (d_model, d_ff, heads) the library carries
-    KERNELS = {"auto": 0, "quad": 1, "board": 2}   # enum bf_kernel
+    KERNELS = {"auto": 0, "quad": 1, "board": 2, "twin": 3}   # enum bf_kernel
     ACC_DTYPES = ("fp16", "fp32")
     n_value = 1
     vmode = 0
@@ -368,10 +369,11 @@ class FusedEncoder:
         wide = self.d_model != self.D
         if wide and fp8:
             raise NotImplementedError("the 512-wide network runs in int8 only")
-        if wide and kernel == "quad":
-            raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernel only")
-        if fp8 and kernel == "board":
-            raise NotImplementedError("the one-position-per-workgroup kernel runs in int8 only")
+        if wide and kernel in ("quad", "twin"):
+            raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernel "
+                                      "(kernel='board' or 'auto') only")
+        if fp8 and kernel in ("board", "twin"):
+            raise NotImplementedError("the one-position-per-workgroup kernels run in int8 only")
         if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
             raise ValueError("the evaluator implements pre-norm ReLU layers only")
         self.n_value = int(net.value.weight.shape[0]) if net is not None else 1
@@ -405,7 +407,7 @@ class FusedEncoder:
         # kernel (int8; small launches of the 256-wide network and the 512-wide network).
         self.kernel = kernel
         self.wstream = self.fparams = self.board_wstream = self.board_fparams = None
-        if not wide and kernel != "board":
+        if not wide and kernel not in ("board", "twin"):
             wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value,
                                             fmt="e4m3" if self.fp8 else "int8")
             if wstream.size != self._lib.bf_wstream_bytes(C.byref(self._shape)) or \
@@ -426,9 +428,16 @@ class FusedEncoder:
     @property
     def label(self) -> str:
         fmt = "e4m3" if self.fp8 else "int8"
-        per = {"auto": "4 or 1 boards/workgroup by batch size", "quad": "4 boards/workgroup",
-               "board": "1 board/workgroup"}[self.kernel if self.board_wstream is not None and self.wstream is not None
-                                             else ("board" if self.wstream is None else "quad")]
+        names = {"quad": "4 boards/workgroup", "board": "1 board/workgroup",
+                 "twin": "1 board/workgroup, 2 workgroups/CU"}
+        if self.kernel != "auto":
+            per = names[self.kernel]
+        elif self.board_wstream is None:
+            per = names["quad"]
+        elif self.d_model != self.D:
+            per = names["board"]
+        else:
+            per = "1 board/workgroup, 1 or 2 workgroups/CU by batch size"
         return f"{fmt} FFN+QKV+out_proj, {per} (gfx950)"
 
     # -- buffers and checks ---------------------------------------------------
@@ -495,7 +504,7 @@ class FusedEncoder:
         rc = self._lib.bf_kernel_choice(C.byref(a))
         if rc < 0:
             raise RuntimeError(f"bf_kernel_choice failed ({rc}): {self._lib.bf_last_error().decode()}")
-        return {1: "quad", 2: "board"}[rc]
+        return {1: "quad", 2: "board", 3: "twin"}[rc]
 
     def _call(self, args: _Args) -> None:
         rc = self._lib.bf_model_forward(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream))

@@ -34,16 +34,22 @@ enum bf_quant {
     BF_QUANT_E4M3 = 1
 };
 
-/* Two kernels compute the same function.  QUAD evaluates four positions per workgroup (one
- * wavefront each, weights shared through LDS): the throughput kernel for large batches of the
- * 256-wide network.  BOARD evaluates one position per workgroup (the four wavefronts split the
- * model width): a quarter of the latency per position for launches that cannot fill the GPU,
- * and the only kernel for the 512-wide network.  For the 256-wide network their results are
- * bit-identical, so AUTO may pick by batch size. */
+/* Three kernels compute the same function.
+ *   QUAD   four positions per workgroup, one wavefront each, weights shared through LDS; carries
+ *          the e4m3 format and the phase profile (256-wide network).
+ *   BOARD  one position per workgroup, the four wavefronts split the model width; one workgroup
+ *          per compute unit: the lowest latency per position (launches that cannot fill the GPU)
+ *          and the only kernel the 512-wide network fits.
+ *   TWIN   the BOARD decomposition shaped so that two workgroups share a compute unit (each SIMD
+ *          holds two wavefronts that cover each other's waits): the highest throughput
+ *          (256-wide network).
+ * BOARD and TWIN read the same blobs (board_wstream / board_fparams), int8 only.  For the
+ * 256-wide network all three return bit-identical results, so AUTO may pick by batch size. */
 enum bf_kernel {
     BF_KERNEL_AUTO = 0,
     BF_KERNEL_QUAD = 1,
-    BF_KERNEL_BOARD = 2
+    BF_KERNEL_BOARD = 2,
+    BF_KERNEL_TWIN = 3
 };
 
 /* Sizes of one 32-token position, fixed by the position format
@@ -52,7 +58,7 @@ enum bf_kernel {
 #define BF_POLICY 64
 #define BF_PROMO 4
 
-/* Network shape.  Supported: d_model 256, n_heads 8, d_ff 1024 (both kernels, both formats)
+/* Network shape.  Supported: d_model 256, n_heads 8, d_ff 1024 (all kernels; e4m3 on QUAD)
  * and d_model 512, n_heads 16, d_ff 2048 (BOARD kernel, int8); head width 32, any
  * n_layers >= 1, n_value 1 (tanh scalar) or 3 (loss/draw/win classes). */
 typedef struct {
@@ -70,8 +76,8 @@ size_t bf_layer_stride_floats(const bf_shape* s); /* stride of one layer inside 
  * feed-forward hidden activations occupy the register file.  Contents are meaningless
  * between launches; launches that may overlap need separate workspaces. */
 size_t bf_workspace_bytes(const bf_shape* s, int64_t n);
-/* The same two blobs in the BOARD kernel's order (int8 only); 0 for an unsupported shape.
- * That kernel needs no workspace. */
+/* The same two blobs in the order of the BOARD and TWIN kernels (int8 only); 0 for an
+ * unsupported shape.  Those kernels need no workspace. */
 size_t bf_board_wstream_bytes(const bf_shape* s);
 size_t bf_board_fparams_floats(const bf_shape* s);
 
@@ -128,15 +134,16 @@ typedef struct {
     void* workspace;        /* bf_workspace_bytes(shape, n) bytes of device memory (QUAD kernel) */
     size_t workspace_bytes;
     const bf_taps* taps; /* NULL in production */
-    /* the weights packed for the BOARD kernel (NULL: that kernel is not available to this
-     * call); wstream / fparams / workspace may be NULL when only the BOARD kernel can run */
+    /* the weights packed for the BOARD / TWIN kernels (NULL: those kernels are not available
+     * to this call); wstream / fparams / workspace may be NULL when QUAD is not to run */
     const uint8_t* board_wstream;
     const float* board_fparams;
-    int32_t kernel;         /* enum bf_kernel; AUTO: BOARD for the 512-wide network and for
-                             * n <= bf_board_max_n() when its blobs are given, else QUAD */
+    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs and int8: BOARD for the
+                             * 512-wide network and for n <= bf_board_max_n(), TWIN above;
+                             * otherwise QUAD */
 } bf_eval_args;
 
-/* Largest n for which AUTO prefers the BOARD kernel on the 256-wide network. */
+/* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */
 int64_t bf_board_max_n(void);
 /* The kernel AUTO would run for these arguments (enum bf_kernel), or a negative bf_status. */
 int bf_kernel_choice(const bf_eval_args* args);
@@ -197,19 +204,20 @@ const char* bf_profile_phase_name(int i);
  * of [policy(64); promo(4); value(n_value); zeros]), fragment (n, q), lane 32g + o holds
  * the four floats W[32 m + o][32 n + 8 q + 4 g + 0..3].
  *
- * BOARD kernel blobs.  Wave w of a workgroup owns tiles TW*w .. TW*w+TW-1 of the model width
- * (TW = d/128), kc = d/256, halves = d_ff/1024.  board_wstream is, for each wave w, its own
+ * BOARD / TWIN kernel blobs.  Wave w of a workgroup owns tiles TW*w .. TW*w+TW-1 of the model
+ * width (TW = d/128), kc = d/256, steps = d_ff/512.  board_wstream is, for each wave w, its own
  * stream: per layer the 8 KiB blocks (same fragment format as above)
  *     for own head i: Q tile chunks 0..kc-1, K tile chunks, V tile chunks
  *     out-proj: for own tile i: chunks 0..kc-1
- *     for half hh: ffn1: for i = 0..7: hidden tile 32 hh + 8 w + i, chunks 0..kc-1;
- *                  ffn2: for chunk c = 4 hh .. 4 hh + 3: for own tile i: block (tile, c)
- * then d/64 blocks holding head tile w (the fp32 fragments (n, q) in order; zeros for w = 3).
+ *     for step s: ffn1: for i = 0..3: hidden tile 16 s + 4 w + i, chunks 0..kc-1;
+ *                 ffn2: for chunk c = 2 s, 2 s + 1: for own tile i: block (tile, c)
+ * then d/64 blocks holding head tile w (the fp32 fragments (n, q) in order; zeros for w = 3)
+ * and one block of zeros (the weight prefetch reads one block past a wave's last).
  * board_fparams is, for each wave w, per layer: part A  ln1_gamma ln1_beta b_q b_k b_v b_out
  * (own channels, d/4 each) sw_q[TW] sw_k[TW] sw_v[TW] sw_out[TW] (per own tile, padded to 16);
- * part B  ln2_gamma ln2_beta (own) b_ffn1 (own hidden channels: 256 per half) b_ffn2 (own)
- * wsum[d_ff/256][d/4] (int32, own channels) sw_ffn1[8 halves] sw_ffn2[TW] (padded to 32);
- * after the four waves the embedding tables and norm_f as below.
+ * part B  ln2_gamma ln2_beta (own) b_ffn1 (own hidden channels: 128 per step) b_ffn2 (own)
+ * wsum[d_ff/256][d/4] (int32, own channels) sw_ffn1[4 per step, padded to 16] sw_ffn2[TW]
+ * (padded to 16); after the four waves the embedding tables and norm_f as below.
  *
  * fparams (fp32 unless noted), per layer at stride bf_layer_stride_floats() (the layer's
  * parameters zero-padded to a multiple of 4 KiB, because a workgroup copies them to LDS

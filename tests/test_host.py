@@ -65,27 +65,28 @@ def test_kernel_choice_follows_shape_blobs_and_batch_size():
     a.shape = hip_impl._Shape(256, 8, 8, 1024, 1, 1e-5)
     a.wstream = a.fparams = a.board_wstream = a.board_fparams = 16      # only tested for NULL here
     cut = lib.bf_board_max_n()
-    assert 64 <= cut < 4096
-    for n, want in ((1, 2), (cut, 2), (cut + 1, 1), (4096, 1)):
+    assert cut == 256                                                    # one position per compute unit
+    for n, want in ((1, 2), (cut, 2), (cut + 1, 3), (4096, 3)):          # BOARD up to the cut, TWIN above
         a.n = n
         assert lib.bf_kernel_choice(ctypes.byref(a)) == want
-    a.n, a.kernel = 4096, 2
-    assert lib.bf_kernel_choice(ctypes.byref(a)) == 2                    # forced
-    a.n, a.kernel = 1, 1
-    assert lib.bf_kernel_choice(ctypes.byref(a)) == 1
+    for forced in (1, 2, 3):
+        a.n, a.kernel = 4096, forced
+        assert lib.bf_kernel_choice(ctypes.byref(a)) == forced
     a.kernel, a.quant = 0, 1                                            # e4m3: four-per-workgroup kernel only
     assert lib.bf_kernel_choice(ctypes.byref(a)) == 1
-    a.kernel = 2
-    assert lib.bf_kernel_choice(ctypes.byref(a)) == -2
+    for forced in (2, 3):
+        a.kernel = forced
+        assert lib.bf_kernel_choice(ctypes.byref(a)) == -2
     a.kernel, a.quant, a.board_wstream = 0, 0, None                     # no board blobs: always quad
     a.n = 1
     assert lib.bf_kernel_choice(ctypes.byref(a)) == 1
-    a.shape = hip_impl._Shape(512, 16, 16, 2048, 1, 1e-5)
+    a.shape = hip_impl._Shape(512, 16, 16, 2048, 1, 1e-5)               # the 512-wide network: BOARD at any size
     a.board_wstream = 16
     a.n = 100000
     assert lib.bf_kernel_choice(ctypes.byref(a)) == 2
-    a.kernel = 1
-    assert lib.bf_kernel_choice(ctypes.byref(a)) == -2
+    for forced in (1, 3):
+        a.kernel = forced
+        assert lib.bf_kernel_choice(ctypes.byref(a)) == -2
     a.kernel = 7
     assert lib.bf_kernel_choice(ctypes.byref(a)) == -1
 
@@ -101,22 +102,28 @@ def test_board_packing_layout_and_sizes():
         shape = hip_impl._Shape(d, layers, heads, f, 1, 1e-5)
         assert ws.size == lib.bf_board_wstream_bytes(ctypes.byref(shape))
         assert fp.size == lib.bf_board_fparams_floats(ctypes.byref(shape))
-        tw, kc, halves, nt = d // 128, d // 256, f // 1024, d // 32
-        bpw = 3 * tw * kc + tw * kc + halves * (8 * kc + 4 * tw)
-        wave_blocks = layers * bpw + nt // 2
+        tw, kc, steps, nt = d // 128, d // 256, f // 512, d // 32
+        bpw = 3 * tw * kc + tw * kc + steps * (4 * kc + 2 * tw)
+        wave_blocks = layers * bpw + nt // 2 + 1                      # + one block of padding
         assert ws.size == 4 * wave_blocks * 8192
+        assert (ws[(3 * wave_blocks - 1) * 8192:3 * wave_blocks * 8192] == 0).all()
         # wave 2, layer 1, first block: Q tile of its first head (tile 2 tw), chunk 0
         q_qkv, s_qkv = hip_impl.quantise_weights_int8(sd["encoder.layers.1.self_attn.in_proj_weight"])
         blk = ws[(2 * wave_blocks + bpw) * 8192:][:8192].view(np.int8).reshape(8, 64, 16)
         assert blk[3, 40, 9] == q_qkv[32 * 2 * tw + 8, 32 * 3 + 8 * 2 + 4 + 1]
-        # its last block of the layer: ffn2 tile 2 tw + tw - 1, chunk 4 halves - 1
+        # its last block of the layer: ffn2 tile 2 tw + tw - 1, last chunk
         q_ff2, s_ff2 = hip_impl.quantise_weights_int8(sd["encoder.layers.1.linear2.weight"])
         blk = ws[(2 * wave_blocks + 2 * bpw - 1) * 8192:][:8192].view(np.int8).reshape(8, 64, 16)
-        assert blk[0, 1, 0] == q_ff2[32 * (3 * tw - 1) + 1, 256 * (4 * halves - 1)]
+        assert blk[0, 1, 0] == q_ff2[32 * (3 * tw - 1) + 1, 256 * (2 * steps - 1)]
+        # first feed-forward block of step 1: hidden tile 16 + 4 * 2, chunk 0
+        q_ff1, s_ff1 = hip_impl.quantise_weights_int8(sd["encoder.layers.1.linear1.weight"])
+        k_ff = 4 * tw * kc + (4 * kc + 2 * tw)
+        blk = ws[(2 * wave_blocks + bpw + k_ff) * 8192:][:8192].view(np.int8).reshape(8, 64, 16)
+        assert blk[1, 33, 2] == q_ff1[32 * 24 + 1, 32 + 4 + 2]
         # parameter slice of wave 2, layer 1
         cw = 32 * tw
         a_floats = 6 * cw + 16
-        b_floats = 3 * cw + 256 * halves + (f // 256) * cw + 32
+        b_floats = 3 * cw + 128 * steps + (f // 256) * cw + 32
         pw = a_floats + b_floats
         sl = fp[(2 * layers + 1) * pw:(2 * layers + 2) * pw]
         own = slice(2 * cw, 3 * cw)
@@ -124,10 +131,12 @@ def test_board_packing_layout_and_sizes():
         assert (sl[4 * cw:5 * cw] == sd["encoder.layers.1.self_attn.in_proj_bias"].numpy()[2 * d:][own]).all()
         assert sl[6 * cw + 2 * tw] == s_qkv[(2 * d + 32 * 2 * tw) // 128]            # sw_v of its first head
         pb = sl[a_floats:]
-        assert (pb[2 * cw:2 * cw + 256] == sd["encoder.layers.1.linear1.bias"].numpy()[512:768]).all()
-        wsum = pb[3 * cw + 256 * halves:][: (f // 256) * cw].view(np.int32).reshape(f // 256, cw)
+        b1 = sd["encoder.layers.1.linear1.bias"].numpy()
+        assert (pb[2 * cw:2 * cw + 128] == b1[256:384]).all() and (pb[2 * cw + 128:2 * cw + 256] == b1[768:896]).all()
+        wsum = pb[3 * cw + 128 * steps:][: (f // 256) * cw].view(np.int32).reshape(f // 256, cw)
         assert (wsum[3] == 128 * q_ff2[own, 768:1024].astype(np.int32).sum(1)).all()
-        assert pb[b_floats - 32 + 8 * halves + 1] == s_ff2[(32 * (2 * tw + 1)) // 128]
+        assert pb[b_floats - 32 + 5] == s_ff1[(512 + 256 + 32) // 128]               # step 1, its second hidden tile
+        assert pb[b_floats - 32 + 16 + 1] == s_ff2[(32 * (2 * tw + 1)) // 128]
         tail = fp[4 * layers * pw:]
         assert (tail[:64 * d] == sd["emb_square.weight"].numpy().reshape(-1)).all() and tail.size == (64 + 12 + 4 + 101 + 3 + 2) * d
 

@@ -1,11 +1,13 @@
-"""Parity of the one-position-per-workgroup kernel, through the C-ABI.
+"""Parity of the one-position-per-workgroup kernels (one and two workgroups per compute unit),
+through the C-ABI.
 
 Same bar as tests/test_parity_gpu.py: operand bytes, int32 accumulators, residual stream, logits,
-value and masked argmax bit-identical to the C checker.  For the 256-wide network the kernel must
-also return exactly what the four-positions-per-workgroup kernel returns (the library picks
-between them by batch size, and a position's result may not depend on the batch it is in); for the
+value and masked argmax bit-identical to the C checker.  For the 256-wide network the kernels
+must also return exactly what the four-positions-per-workgroup kernel returns (the library picks
+among them by batch size, and a position's result may not depend on the batch it is in); for the
 512-wide, 16-head, 16-layer network (two 256-deep k-chunks per matmul of the width, eight for the
-second feed-forward matmul, summed in float64) it is the only kernel.
+second feed-forward matmul, summed in float64) the one-workgroup-per-compute-unit form is the
+only kernel.
 """
 import numpy as np
 import pytest
@@ -31,7 +33,7 @@ def _make(d, heads, layers, nv=1, seed=0):
 @pytest.fixture(scope="module")
 def base():
     net, sd = _make(256, 8, 8)
-    return (net, sd, encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="board"),
+    return (net, sd, {k: encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=k) for k in ("board", "twin")},
             encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="quad"), c_oracle.COracle(sd))
 
 
@@ -53,8 +55,10 @@ def _bits_equal(a: torch.Tensor, b: np.ndarray) -> bool:
                                         == b.view(np.int32 if b.dtype == np.float32 else b.dtype)).all())
 
 
-def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base):
-    net, sd, board, quad, co = base
+@pytest.mark.parametrize("kernel", ["board", "twin"])
+def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base, kernel):
+    net, sd, boards, quad, co = base
+    board = boards[kernel]
     b, c, r, m = positions.random_positions(48, plies=120, seed=11, stamp_queen=True)
     got = board.forward_taps(*_dev(b, c, r), mask=m.cuda())
     want = co.forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy(), taps=True)
@@ -62,13 +66,15 @@ def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base):
         assert _bits_equal(got[k], want[k]), k
 
 
+@pytest.mark.parametrize("kernel", ["board", "twin"])
 @pytest.mark.parametrize("nv", [1, 3])
-def test_the_two_kernels_return_the_same_bits(base, nv):
+def test_the_kernels_return_the_same_bits(base, nv, kernel):
     if nv == 1:
-        net, sd, board, quad, co = base
+        net, sd, boards, quad, co = base
+        board = boards[kernel]
     else:
         net, sd = _make(256, 8, 8, nv=3, seed=5)
-        board = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="board")
+        board = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=kernel)
         quad = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="quad")
     b, c, r, m = positions.random_positions(301, plies=120, seed=21)           # odd on purpose
     bd, cd, rd, md = _dev(b, c, r, m)
@@ -80,7 +86,7 @@ def test_the_two_kernels_return_the_same_bits(base, nv):
     assert torch.equal(board.forward_full(bd, cd, rd)[0], raw_q) and torch.isfinite(raw_q).all()
     one = board.forward_full(bd[7:8], cd[7:8], rd[7:8])[0]
     assert torch.equal(one, raw_q[7:8])
-    half_b = encoder_impl("hip")(net, int8=True, kernel="board").forward_full(bd, cd, rd)[0]
+    half_b = encoder_impl("hip")(net, int8=True, kernel=kernel).forward_full(bd, cd, rd)[0]
     assert half_b.dtype is torch.float16 and torch.equal(half_b, raw_q.half())
     # teacher-forced single layers and the heads alone agree as well
     x = torch.randn(301, 32, 256, generator=torch.Generator().manual_seed(3)).cuda()
@@ -92,22 +98,45 @@ def test_the_two_kernels_return_the_same_bits(base, nv):
 
 
 def test_automatic_choice_switches_kernel_by_batch_size_without_changing_results(base):
-    net, sd, board, quad, co = base
+    net, sd, boards, quad, co = base
     auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
     cut = int(auto._lib.bf_board_max_n())
     assert auto.kernel_choice(1) == "board" and auto.kernel_choice(cut) == "board"
-    assert auto.kernel_choice(cut + 1) == "quad" and auto.kernel_choice(4096) == "quad"
+    assert auto.kernel_choice(cut + 1) == "twin" and auto.kernel_choice(4096) == "twin"
     assert "by batch size" in auto.label
     b, c, r, m = positions.random_positions(cut + 4, plies=120, seed=22)
     bd, cd, rd, md = _dev(b, c, r, m)
-    big = [t.clone() for t in auto.forward_masked(bd, cd, rd, md)]                        # quad
-    small = auto.forward_masked(bd[:cut], cd[:cut], rd[:cut], md[:cut])                  # board
+    big = [t.clone() for t in auto.forward_masked(bd, cd, rd, md)]                        # two workgroups per CU
+    small = auto.forward_masked(bd[:cut], cd[:cut], rd[:cut], md[:cut])                  # one
     for x, y in zip(big, small):
         assert torch.equal(x[:cut], y)
+    ref = quad.forward_masked(bd, cd, rd, md)
+    for x, y in zip(big, ref):
+        assert torch.equal(x, y)
     fp8 = encoder_impl("hip")(net, fp8=True)
-    assert fp8.kernel_choice(1) == "quad"
-    with pytest.raises(NotImplementedError):
-        encoder_impl("hip")(net, fp8=True, kernel="board")
+    assert fp8.kernel_choice(1) == "quad" and fp8.kernel_choice(4096) == "quad"
+    for k in ("board", "twin"):
+        with pytest.raises(NotImplementedError):
+            encoder_impl("hip")(net, fp8=True, kernel=k)
+
+
+def test_full_batch_at_4096_on_the_throughput_kernel(base):
+    net, sd, boards, quad, co = base
+    auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
+    assert auto.kernel_choice(4096) == "twin"
+    b, c, r, m = positions.random_positions(4096, plies=120, seed=0)
+    bd, cd, rd, md = _dev(b, c, r, m)
+    p, q, v, best = [t.clone() for t in auto.forward_masked(bd, cd, rd, md)]
+    idx = np.arange(3, 4096, 41)
+    want = co.forward(b.numpy()[idx], c.numpy()[idx], r.numpy()[idx], mask=m.numpy()[idx])
+    assert _bits_equal(p[idx], want["policy"]) and _bits_equal(q[idx], want["promo"])
+    assert _bits_equal(v[idx], want["value"]) and (best.cpu().numpy()[idx] == want["best"]).all()
+    ref = quad.forward_masked(bd, cd, rd, md)
+    assert torch.equal(p, ref[0]) and torch.equal(q, ref[1]) and torch.equal(v, ref[2]) and torch.equal(best, ref[3])
+    again = auto.forward_masked(bd, cd, rd, md)
+    assert torch.equal(again[0], p) and torch.equal(again[3], best)                       # deterministic
+    legal = ((md[..., None] >> torch.arange(64, device="cuda")) & 1).bool()
+    assert torch.isneginf(p[~legal]).all() and torch.isfinite(p[legal]).all() and (v.abs() <= 1).all()
 
 
 def test_stress_network_bit_exact_against_the_c_checker_with_every_tap(stress):
@@ -145,8 +174,9 @@ def test_stress_network_bit_exact_against_the_c_checker_with_every_tap(stress):
     assert torch.equal(heads["policy"], got["policy"]) and torch.equal(heads["value"], got["value"])
     with pytest.raises(NotImplementedError):
         encoder_impl("hip")(net, fp8=True)
-    with pytest.raises(NotImplementedError):
-        encoder_impl("hip")(net, int8=True, kernel="quad")
+    for k in ("quad", "twin"):
+        with pytest.raises(NotImplementedError):
+            encoder_impl("hip")(net, int8=True, kernel=k)
 
 
 def test_stress_network_win_draw_loss_head_and_full_batch_properties():
