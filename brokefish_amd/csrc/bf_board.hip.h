@@ -21,7 +21,7 @@
 //                 wave, so every SIMD holds two wavefronts of different positions and one's
 //                 waits (LDS round trips, barriers, MFMA results) are covered by the other's
 //                 work.  Weight fragments go from L2 straight to registers (half a block = four
-//                 fragments at a time, prefetched one block ahead through three register sets).
+//                 fragments at a time, prefetched through a rotation of register sets).
 //                 Highest throughput.
 //
 // LDS map (bytes): [ring: 4 waves x SLOTS x 8 KiB, absent in the TWIN form] [xch: 3 KiB]
@@ -30,6 +30,16 @@
 #pragma once
 
 #include "bf_device.hip.h"
+
+// TWIN form: workgroups per compute unit, and register sets of the weight prefetch (one set =
+// half a block; SETS - 1 half-blocks are in flight).  Measured on MI355X at batch 4096: three
+// workgroups per unit spill too much (1.42 M evals/s against 2.10 M), four sets beat three by 2 %.
+#ifndef BF_TWIN_SETS
+#define BF_TWIN_SETS 4
+#endif
+#ifndef BF_TWIN_OCC
+#define BF_TWIN_OCC 2
+#endif
 
 namespace bf {
 namespace board {
@@ -45,10 +55,10 @@ struct Cfg : Layout<DM> {
     static constexpr int ACT_OFF = HID_OFF + 16 * FRAG;
     static constexpr int PAR_OFF = ACT_OFF + L::NT * FRAG;
     static constexpr int LDS_BYTES = PAR_OFF + 4 * L::PW_FLOATS * 4;
-    static_assert(LDS_BYTES <= (TWIN ? 80 : 160) * 1024, "LDS budget: one or two workgroups per compute unit");
+    static_assert(LDS_BYTES <= (TWIN ? 160 / BF_TWIN_OCC : 160) * 1024, "LDS budget: one or two workgroups per compute unit");
     static_assert(L::NT * 4 * FRAG <= LDS_BYTES - HID_OFF, "normalised stream overlay");
     static_assert(L::BPW % L::SLOTS == 0, "ring slot of a block must not depend on the layer");
-    static_assert((2 * L::BPW) % 3 == 0, "register set of a half-block must not depend on the layer");
+    static_assert((2 * L::BPW) % BF_TWIN_SETS == 0, "register set of a half-block must not depend on the layer");
 };
 
 // workgroup barrier that waits for this wave's LDS traffic only (outstanding direct-to-LDS
@@ -92,11 +102,12 @@ __device__ __forceinline__ float chunk_sum(const v16i (&acc)[KC], int i, const f
 }
 
 template <int DM, bool TAPS, bool TWIN>
-__global__ __launch_bounds__(THREADS, TWIN ? 2 : 1) void board_kernel(const KArgs a) {
+__global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(const KArgs a) {
     typedef Cfg<DM, TWIN> C;
     constexpr int D = C::D, F = C::F, NT = C::NT, TW = C::TW, CW = C::CW, KC = C::KC, KCF = C::KCF;
     constexpr int STEPS = C::STEPS, BPW = C::BPW, HB = C::HB, SLOTS = C::SLOTS, WPC = 4 / KC;
     constexpr int HALF = BLOCK / 2;   // four fragments: the unit of the register prefetch (TWIN)
+    constexpr int NSETS = BF_TWIN_SETS;   // register sets of the prefetch: NSETS - 1 half-blocks in flight
     constexpr int VM_AHEAD = TAPS ? 0 : (SLOTS - 1) * 8;   // ring loads that may stay in flight at a ring wait
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -117,7 +128,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? 2 : 1) void board_kernel(const KArg
     const float* const gp = a.fparams + (size_t)4 * a.n_layers * C::PW_FLOATS;       // tables, final norm
 
     // TWIN: half-block `hseq` of this wave's stream (consumption order) into register set `set`
-    v4i frt[3][4];
+    v4i frt[NSETS][4];
     auto load_half = [&](int hseq, int set) {
         const uint8_t* src = wsrc + (size_t)hseq * HALF;
 #pragma unroll
@@ -216,8 +227,8 @@ __global__ __launch_bounds__(THREADS, TWIN ? 2 : 1) void board_kernel(const KArg
 
     // ---- start the weight stream and the first layer's parameters ------------------------------
     if constexpr (TWIN) {
-        load_half(0, 0);
-        load_half(1, 1);
+#pragma unroll
+        for (int j = 0; j < NSETS - 1; j++) load_half(j, j);
     } else {
 #pragma unroll
         for (int j = 0; j < SLOTS; j++) issue_block(j, j);
@@ -287,8 +298,8 @@ __global__ __launch_bounds__(THREADS, TWIN ? 2 : 1) void board_kernel(const KArg
         const size_t bl = (size_t)b * nl_run + li;   // tap row
         const int lnext = l + 1 < a.l1 ? l + 1 : l;  // after the last layer the same slice is fetched again
         // Multiply by block k of this wave's layer.
-        // TWIN: its two halves sit in register sets 2k % 3 and (2k + 1) % 3; each half's set is
-        // refilled with the half three positions on once consumed.
+        // TWIN: its two halves sit in register sets 2k % NSETS and (2k + 1) % NSETS; a set is refilled
+        // with the half-block NSETS positions on once it has been consumed.
         // !TWIN: the block is in `fr`; the ring slot it came from is refilled SLOTS blocks ahead,
         // then block k+1 is read from its slot.
         const int hbase = li * 2 * BPW;
@@ -297,14 +308,14 @@ __global__ __launch_bounds__(THREADS, TWIN ? 2 : 1) void board_kernel(const KArg
         const v4i* act_ = (actp);                                                                    \
         v16i r_ = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};                                  \
         if constexpr (TWIN) {                                                                        \
-            load_half(hbase + 2 * (k) + 2, (2 * (k) + 2) % 3);                                       \
+            load_half(hbase + 2 * (k) + NSETS - 1, (2 * (k) + NSETS - 1) % NSETS);                   \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
-                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[s_], frt[(2 * (k)) % 3][s_], r_, 0, 0, 0)  \
-                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(frt[(2 * (k)) % 3][s_], act_[s_], r_, 0, 0, 0); \
-            load_half(hbase + 2 * (k) + 3, (2 * (k) + 3) % 3);                                       \
+                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[s_], frt[(2 * (k)) % NSETS][s_], r_, 0, 0, 0)  \
+                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(frt[(2 * (k)) % NSETS][s_], act_[s_], r_, 0, 0, 0); \
+            load_half(hbase + 2 * (k) + NSETS, (2 * (k) + NSETS) % NSETS);                           \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
-                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[4 + s_], frt[(2 * (k) + 1) % 3][s_], r_, 0, 0, 0)  \
-                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(frt[(2 * (k) + 1) % 3][s_], act_[4 + s_], r_, 0, 0, 0); \
+                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[4 + s_], frt[(2 * (k) + 1) % NSETS][s_], r_, 0, 0, 0)  \
+                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(frt[(2 * (k) + 1) % NSETS][s_], act_[4 + s_], r_, 0, 0, 0); \
         } else {                                                                                     \
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                       \
             issue_block(li * BPW + (k) + SLOTS, (k) % SLOTS);                                        \
@@ -584,8 +595,8 @@ __global__ __launch_bounds__(THREADS, TWIN ? 2 : 1) void board_kernel(const KArg
     wait_vm<0>();   // also: no parameter copy is still landing where the normalised stream goes
     if (a.l1 != a.n_layers) {
         if constexpr (TWIN) {
-            load_half(2 * hseq0, 0);
-            load_half(2 * hseq0 + 1, 1);
+#pragma unroll
+            for (int j = 0; j < NSETS - 1; j++) load_half(2 * hseq0 + j, j);
         } else {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
@@ -618,10 +629,11 @@ __global__ __launch_bounds__(THREADS, TWIN ? 2 : 1) void board_kernel(const KArg
     if constexpr (TWIN) {
 #pragma unroll
         for (int hi = 0; hi < 2 * HB; hi++) {          // half-block = the four fragments (n = hi, q = 0..3)
-            load_half(2 * hseq0 + hi + 2, (hi + 2) % 3);   // the stream is padded by one block
+            // the stream is padded by one block: two half-blocks past the last head block exist
+            if (hi + NSETS - 1 < 2 * HB + 2) load_half(2 * hseq0 + hi + NSETS - 1, (hi + NSETS - 1) % NSETS);
 #pragma unroll
             for (int s = 0; s < 4; s++) {
-                const v4f w = __builtin_bit_cast(v4f, frt[hi % 3][s]);
+                const v4f w = __builtin_bit_cast(v4f, frt[hi % NSETS][s]);
                 const v4f hv = *reinterpret_cast<const v4f*>(hnb + ((hi * 4 + s) * 64 + lane) * 4);
 #pragma unroll
                 for (int k = 0; k < 4; k++) head = __builtin_amdgcn_mfma_f32_32x32x2f32(w[k], hv[k], head, 0, 0, 0);
