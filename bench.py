@@ -24,9 +24,10 @@ if ROOT not in sys.path:
 OPS_PER_EVAL = 402_653_184            # 2 * 32 tokens * 8 layers * 12 * 256^2 int8 ops in the weight GEMMs
 OPS_PER_EVAL_STRESS = 3_221_225_472   # 2 * 32 tokens * 16 layers * 12 * 512^2 (the 512-wide, 16-layer network)
 PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s (dense fp8 MFMA: the same figure)
-# HBM bytes per launch of the default workload (batch 4096), from the FETCH_SIZE / WRITE_SIZE
-# counter runs summarised in profiles/eval_kernel_int8_batch4096.md (calibrated on a 1 GiB copy).
-MEASURED_TRAFFIC_BYTES = {4096: 3.07e9}
+# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/
+# (calibrated on a 1 GiB copy), by (network shape, kernel, batch).
+MEASURED_TRAFFIC_BYTES = {("base", "twin", 4096): 1.00e9, ("base", "quad", 4096): 3.07e9,
+                          ("base", "board", 256): 5.5e7, ("stress", "board", 16384): 2.66e10}
 
 
 def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0, mode: str = "int8"):
@@ -130,7 +131,7 @@ def main() -> int:
                                "fp16 logits out, seed-0 random-init weights"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_OPS / 1e12, "unit": "TOP/s",
                      "frac": achieved / (PEAK_INT8_OPS / 1e12),
-                     "traffic": None if (fp8 or stress or model.kernel_choice(a.batch) != "quad") else MEASURED_TRAFFIC_BYTES.get(a.batch),
+                     "traffic": None if fp8 else MEASURED_TRAFFIC_BYTES.get((a.shape, model.kernel_choice(a.batch), a.batch)),
                      "kernel_ms": kern_ms, "ops_per_launch": ops_per_eval * a.batch},
     }
     if a.sweep:
