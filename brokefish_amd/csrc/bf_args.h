@@ -130,5 +130,7 @@ hipError_t launch_board512_taps(const KArgs& k, hipStream_t stream);
 // the same with two workgroups per compute unit (256-wide network)
 hipError_t launch_twin256(const KArgs& k, hipStream_t stream);
 hipError_t launch_twin256_taps(const KArgs& k, hipStream_t stream);
+hipError_t launch_twin256_fp8(const KArgs& k, hipStream_t stream);
+hipError_t launch_twin256_fp8_taps(const KArgs& k, hipStream_t stream);
 
 }  // namespace bf

@@ -87,12 +87,28 @@ __device__ __forceinline__ void dma(const float* src, float* dst, int nfloats, i
                                          (__attribute__((address_space(3))) void*)(d + full * FRAG), 16, 0, 0);
 }
 
+// one 16-byte fragment step of a block product: a 32-deep int8 MFMA, or two 16-deep e4m3 MFMAs
+template <bool SWAP>
+__device__ __forceinline__ v16i frag_mma(const v4i& w, const v4i& act, const v16i& acc) {
+    return SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act, w, acc, 0, 0, 0)
+                : __builtin_amdgcn_mfma_i32_32x32x32_i8(w, act, acc, 0, 0, 0);
+}
+template <bool SWAP>
+__device__ __forceinline__ v16f frag_mma(const v4i& w, const v4i& act, v16f acc) {
+    const v2l wl = __builtin_bit_cast(v2l, w), al = __builtin_bit_cast(v2l, act);
+#pragma unroll
+    for (int h = 0; h < 2; h++)
+        acc = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[h], wl[h], acc, 0, 0, 0)
+                   : __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(wl[h], al[h], acc, 0, 0, 0);
+    return acc;
+}
+
 // acc * sa summed over the k-chunks in float64, cast once (one chunk: the fp32 product, which
 // is the same number)
-template <int KC>
-__device__ __forceinline__ float chunk_sum(const v16i (&acc)[KC], int i, const float (&sa)[KC]) {
+template <int KC, typename ACC>
+__device__ __forceinline__ float chunk_sum(const ACC (&acc)[KC], int i, const float (&sa)[KC]) {
     if constexpr (KC == 1) {
-        return (float)acc[0][i] * sa[0];
+        return accf(acc[0], i) * sa[0];
     } else {
         double o = (double)acc[0][i] * (double)sa[0];
 #pragma unroll
@@ -101,9 +117,11 @@ __device__ __forceinline__ float chunk_sum(const v16i (&acc)[KC], int i, const f
     }
 }
 
-template <int DM, bool TAPS, bool TWIN>
+template <int DM, bool TAPS, bool TWIN, bool FP8>
 __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(const KArgs a) {
     typedef Cfg<DM, TWIN> C;
+    typedef typename Acc<FP8>::type acc_t;
+    static_assert(!FP8 || DM == 256, "e4m3: one k-chunk per matmul of the width (fp32 sums over the chunks of ffn2 only)");
     constexpr int D = C::D, F = C::F, NT = C::NT, TW = C::TW, CW = C::CW, KC = C::KC, KCF = C::KCF;
     constexpr int STEPS = C::STEPS, BPW = C::BPW, HB = C::HB, SLOTS = C::SLOTS, WPC = 4 / KC;
     constexpr int HALF = BLOCK / 2;   // four fragments: the unit of the register prefetch (TWIN)
@@ -204,7 +222,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
 #pragma unroll
             for (int w = c * WPC; w < (c + 1) * WPC; w++) m = __builtin_fmaxf(m, xch[2 * 256 + w * 64 + lane]);
             m = __builtin_fmaxf(m, partner(m, g));
-            sa[c] = m > 0.0f ? m / 127.0f : 1.0f;
+            sa[c] = m > 0.0f ? m / (FP8 ? 8.0f : 127.0f) : 1.0f;
         }
         const float so = KC == 1 ? sa[0] : (wave < WPC ? sa[0] : sa[KC - 1]);
         const float inv = 1.0f / so;
@@ -213,7 +231,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             v4i w;
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                w[j] = (int)quant4<false>(y[i][4 * j], y[i][4 * j + 1], y[i][4 * j + 2], y[i][4 * j + 3], so, inv);
+                w[j] = (int)quant4<FP8>(y[i][4 * j], y[i][4 * j + 1], y[i][4 * j + 2], y[i][4 * j + 3], so, inv);
             *reinterpret_cast<v4i*>(act + (TW * wave + i) * FRAG + lane * 16) = w;
             if (TAPS && tap)
 #pragma unroll
@@ -304,24 +322,21 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
         // then block k+1 is read from its slot.
         const int hbase = li * 2 * BPW;
 #define BF_WMM(SWAP, k, actp)                                                                        \
-    ([&]() -> v16i {                                                                                 \
+    ([&]() -> acc_t {                                                                                \
         const v4i* act_ = (actp);                                                                    \
-        v16i r_ = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};                                  \
+        acc_t r_ = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};                                 \
         if constexpr (TWIN) {                                                                        \
             load_half(hbase + 2 * (k) + NSETS - 1, (2 * (k) + NSETS - 1) % NSETS);                   \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
-                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[s_], frt[(2 * (k)) % NSETS][s_], r_, 0, 0, 0)  \
-                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(frt[(2 * (k)) % NSETS][s_], act_[s_], r_, 0, 0, 0); \
+                r_ = frag_mma<SWAP>(frt[(2 * (k)) % NSETS][s_], act_[s_], r_);                       \
             load_half(hbase + 2 * (k) + NSETS, (2 * (k) + NSETS) % NSETS);                           \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
-                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[4 + s_], frt[(2 * (k) + 1) % NSETS][s_], r_, 0, 0, 0)  \
-                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(frt[(2 * (k) + 1) % NSETS][s_], act_[4 + s_], r_, 0, 0, 0); \
+                r_ = frag_mma<SWAP>(frt[(2 * (k) + 1) % NSETS][s_], act_[4 + s_], r_);               \
         } else {                                                                                     \
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                       \
             issue_block(li * BPW + (k) + SLOTS, (k) % SLOTS);                                        \
             _Pragma("unroll") for (int s_ = 0; s_ < 8; s_++)                                         \
-                r_ = SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act_[s_], fr[s_], r_, 0, 0, 0)     \
-                          : __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[s_], act_[s_], r_, 0, 0, 0);    \
+                r_ = frag_mma<SWAP>(fr[s_], act_[s_], r_);                                           \
             wait_vm<VM_AHEAD>();                                                                     \
             read_slot(((k) + 1) % SLOTS);                                                            \
         }                                                                                            \
@@ -346,7 +361,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
         // !TWIN: software-pipelined -- the three weight GEMMs of head i+1 are issued right after the
         // score MFMAs of head i, so the matrix pipe works through them under head i's softmax.
         float o[TW][16];
-        v16i accq[KC], acck[KC], accv[KC];
+        acc_t accq[KC], acck[KC], accv[KC];
 #pragma unroll
         for (int i = 0; i < TW; i++) {
             if (TWIN || i == 0) {
@@ -385,9 +400,9 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
                             int* row = a.taps.acc_qkv + ((bl * KC + c) * T + t) * 3 * D;
-                            row[32 * h + ch(r, g)] = accq[c][r];
-                            row[D + 32 * h + ch(r, g)] = acck[c][r];
-                            a.taps.acc_qkv[((bl * KC + c) * T + ch(r, g)) * 3 * D + 2 * D + 32 * h + t] = accv[c][r];
+                            row[32 * h + ch(r, g)] = accbits(accq[c], r);
+                            row[D + 32 * h + ch(r, g)] = accbits(acck[c], r);
+                            a.taps.acc_qkv[((bl * KC + c) * T + ch(r, g)) * 3 * D + 2 * D + 32 * h + t] = accbits(accv[c], r);
                         }
             }
             // scores, transposed: lane = query token, register r = key ch(r, g)
@@ -432,7 +447,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             float so[KC];
             quant_exchange(o, so, oq, TAPS ? a.taps.qa_out : nullptr, bl);
             constexpr int K0 = 3 * KC * TW;
-            v16i acc2[2][KC];
+            acc_t acc2[2][KC];
 #pragma unroll
             for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, K0 + c, &oq[8 * c]);
 #pragma unroll
@@ -454,7 +469,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
                     for (int c = 0; c < KC; c++)
 #pragma unroll
                         for (int r = 0; r < 16; r++)
-                            a.taps.acc_out[((bl * KC + c) * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = acc2[i & 1][c][r];
+                            a.taps.acc_out[((bl * KC + c) * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = accbits(acc2[i & 1][c], r);
             }
         }
         // the attention-phase parameters are dead: fetch the next layer's
@@ -467,7 +482,8 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             layernorm(x, pB + C::B_LN2G, pB + C::B_LN2B, y);
             quant_exchange(y, sa, xq, TAPS ? a.taps.qa_ff1 : nullptr, bl);
         }
-        double o64[TW][16];
+        double o64[TW][16];   // int8: float64 sums over the k-chunks
+        float o32[TW][16];    // e4m3: fp32 sums over the k-tiles
         constexpr int KF = 3 * KC * TW + KC * TW;   // first feed-forward block of the layer
 #pragma unroll
         for (int st = 0; st < STEPS; st++) {
@@ -477,7 +493,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             {
                 float hf[4][16];
                 float am = 0.0f;
-                v16i acc2[2][KC];
+                acc_t acc2[2][KC];
 #pragma unroll
                 for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + c, &xq[8 * c]);
 #pragma unroll
@@ -502,17 +518,18 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
                         for (int c = 0; c < KC; c++)
 #pragma unroll
                             for (int r = 0; r < 16; r++)
-                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * wave + 32 * i + ch(r, g)] = acc2[i & 1][c][r];
+                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * wave + 32 * i + ch(r, g)] = accbits(acc2[i & 1][c], r);
                 }
-                // unsigned quantiser over the 256-wide chunk this wave shares with its neighbour (waves
-                // 0,1: first chunk of the step; 2,3: second); bytes stored as q - 128 for the signed MFMA
+                // quantiser over the 256-wide chunk this wave shares with its neighbour (waves 0,1: first
+                // chunk of the step; 2,3: second).  int8: unsigned, bytes stored as q - 128 for the signed
+                // MFMA; e4m3: the ordinary signed quantiser (the values are non-negative)
                 xch[2 * 256 + wave * 64 + lane] = am;
                 lds_barrier();
 #pragma unroll
                 for (int c = 0; c < 2; c++) {
                     float m = __builtin_fmaxf(xch[2 * 256 + (2 * c) * 64 + lane], xch[2 * 256 + (2 * c + 1) * 64 + lane]);
                     m = __builtin_fmaxf(m, partner(m, g));
-                    sh[c] = m > 0.0f ? m / 255.0f : 1.0f;
+                    sh[c] = m > 0.0f ? m / (FP8 ? 8.0f : 255.0f) : 1.0f;
                 }
                 const float s8 = wave < 2 ? sh[0] : sh[1];
                 const float inv = 1.0f / s8;
@@ -521,10 +538,10 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
                     v4i w;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        const unsigned u = quant4<false>(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
+                        const unsigned u = quant4<FP8>(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
                         if (TAPS && a.taps.qa_ff2)
                             *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 512 * st + 128 * wave + 32 * i + 8 * j + 4 * g) = u;
-                        w[j] = (int)(u ^ 0x80808080u);
+                        w[j] = (int)(FP8 ? u : (u ^ 0x80808080u));
                     }
                     *reinterpret_cast<v4i*>(hid + (4 * wave + i) * FRAG + lane * 16) = w;
                 }
@@ -533,7 +550,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             // second matmul, chunk-major: one chunk of the hidden row (eight fragments) serves this
             // wave's TW output tiles; the float64 sums over the chunks stay in chunk order
             const int k2 = k1 + 4 * KC;
-            v16i acc2[2];
+            acc_t acc2[2];
             v4i hqc[8];
 #pragma unroll
             for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + s * FRAG + lane * 16);
@@ -541,9 +558,8 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
 #pragma unroll
             for (int idx = 0; idx < 2 * TW; idx++) {
                 const int c = idx / TW, i = idx % TW;
-                const double sc = (double)sh[c];
                 v4i ws[4];
-                load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * i, g, ws);
+                if (!FP8) load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * i, g, ws);
                 if (idx + 1 < 2 * TW) {
                     if ((idx + 1) % TW == 0)
 #pragma unroll
@@ -551,19 +567,33 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
                             hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * (c + 1) + s) * FRAG + lane * 16);
                     acc2[(idx + 1) & 1] = BF_WMM(false, k2 + idx + 1, &hqc[0]);
                 }
-                const v16i acc = acc2[idx & 1];
+                const acc_t acc = acc2[idx & 1];
+                if constexpr (FP8) {
+                    // descale each 256-deep tile with its own scales, fp32 sum over the tiles
+                    const float sw = pB[C::B_SW + 16 + i * KCF + 2 * st + c];
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-#pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        const int full = acc[4 * j + k] + ws[j][k];
-                        o64[i][4 * j + k] = (st == 0 && c == 0) ? (double)full * sc
-                                                                : __builtin_fma((double)full, sc, o64[i][4 * j + k]);
+                    for (int r = 0; r < 16; r++) {
+                        const float part = (accf(acc, r) * sh[c]) * sw;
+                        o32[i][r] = (st == 0 && c == 0) ? part : o32[i][r] + part;
                         if (TAPS && a.taps.acc_ff2)
-                            a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * wave + i) + 8 * j + 4 * g + k] = full;
+                            a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = accbits(acc, r);
                     }
+                    pin16(o32[i]);
+                } else {
+                    const double sc = (double)sh[c];
 #pragma unroll
-                for (int r = 0; r < 16; r++) pin(o64[i][r]);
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int k = 0; k < 4; k++) {
+                            const int full = accbits(acc, 4 * j + k) + ws[j][k];
+                            o64[i][4 * j + k] = (st == 0 && c == 0) ? (double)full * sc
+                                                                    : __builtin_fma((double)full, sc, o64[i][4 * j + k]);
+                            if (TAPS && a.taps.acc_ff2)
+                                a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * wave + i) + 8 * j + 4 * g + k] = full;
+                        }
+#pragma unroll
+                    for (int r = 0; r < 16; r++) pin(o64[i][r]);
+                }
             }
         }
 #pragma unroll
@@ -574,8 +604,12 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int k = 0; k < 4; k++)
-                    x[i][4 * j + k] = x[i][4 * j + k] + ((float)o64[i][4 * j + k] * sw + b2[j][k]);
+                for (int k = 0; k < 4; k++) {
+                    float upd;
+                    if constexpr (FP8) upd = o32[i][4 * j + k] + b2[j][k];
+                    else upd = (float)o64[i][4 * j + k] * sw + b2[j][k];
+                    x[i][4 * j + k] = x[i][4 * j + k] + upd;
+                }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         dma(wpar + (size_t)lnext * C::PW_FLOATS + C::A_FLOATS, pB, C::B_FLOATS, lane);
@@ -735,18 +769,18 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     }
 }
 
-template <int DM, bool TAPS, bool TWIN>
+template <int DM, bool TAPS, bool TWIN, bool FP8 = false>
 hipError_t launch_board(const KArgs& k, hipStream_t stream) {
     // more than 64 KiB of dynamic LDS has to be requested once per kernel (per thread: cheap)
     static thread_local bool lds_set = false;
     constexpr int lds_bytes = Cfg<DM, TWIN>::LDS_BYTES;
     if (!lds_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&board_kernel<DM, TAPS, TWIN>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&board_kernel<DM, TAPS, TWIN, FP8>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess) return e;
         lds_set = true;
     }
-    hipLaunchKernelGGL((board_kernel<DM, TAPS, TWIN>), dim3(k.n), dim3(THREADS), lds_bytes, stream, k);
+    hipLaunchKernelGGL((board_kernel<DM, TAPS, TWIN, FP8>), dim3(k.n), dim3(THREADS), lds_bytes, stream, k);
     return hipGetLastError();
 }
 

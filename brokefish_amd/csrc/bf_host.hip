@@ -98,7 +98,9 @@ static int choose_kernel(const bf_eval_args* a) {
         return fail(BF_ERR_ARGUMENT, "quant must be BF_QUANT_INT8 or BF_QUANT_E4M3");
     const bool have_quad = a->wstream && a->fparams, have_board = a->board_wstream && a->board_fparams;
     const bool quad_can = shape_ok(&a->shape) && have_quad;
+    // the board blobs are packed for one format; BOARD runs int8, TWIN both
     const bool board_can = have_board && a->quant == BF_QUANT_INT8;
+    const bool twin_can = have_board && shape_ok(&a->shape);
     switch (a->kernel) {
     case BF_KERNEL_QUAD:
         if (!quad_can) return fail(BF_ERR_UNSUPPORTED, "the four-positions-per-workgroup kernel needs the 256-wide network and wstream/fparams");
@@ -107,11 +109,12 @@ static int choose_kernel(const bf_eval_args* a) {
         if (!board_can) return fail(BF_ERR_UNSUPPORTED, "the one-position-per-workgroup kernel needs board_wstream/board_fparams and the int8 format");
         return BF_KERNEL_BOARD;
     case BF_KERNEL_TWIN:
-        if (!board_can || !shape_ok(&a->shape))
-            return fail(BF_ERR_UNSUPPORTED, "the two-workgroups-per-compute-unit kernel needs the 256-wide network, board_wstream/board_fparams and the int8 format");
+        if (!twin_can)
+            return fail(BF_ERR_UNSUPPORTED, "the two-workgroups-per-compute-unit kernel needs the 256-wide network and board_wstream/board_fparams");
         return BF_KERNEL_TWIN;
     case BF_KERNEL_AUTO:
-        if (board_can) return (shape_ok(&a->shape) && a->n > kBoardMaxN) ? BF_KERNEL_TWIN : BF_KERNEL_BOARD;
+        if (board_can) return (twin_can && a->n > kBoardMaxN) ? BF_KERNEL_TWIN : BF_KERNEL_BOARD;
+        if (twin_can) return BF_KERNEL_TWIN;      // e4m3
         if (quad_can) return BF_KERNEL_QUAD;
         return fail(BF_ERR_ARGUMENT, shape512(&a->shape)
                         ? "the 512-wide network runs on the one-position-per-workgroup kernel: int8, board_wstream/board_fparams required"
@@ -165,7 +168,10 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream
     hipError_t e;
     if (kind == BF_KERNEL_TWIN) {
         if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
-        e = a->taps ? bf::launch_twin256_taps(k, stream) : bf::launch_twin256(k, stream);
+        if (a->quant == BF_QUANT_E4M3)
+            e = a->taps ? bf::launch_twin256_fp8_taps(k, stream) : bf::launch_twin256_fp8(k, stream);
+        else
+            e = a->taps ? bf::launch_twin256_taps(k, stream) : bf::launch_twin256(k, stream);
     } else if (kind == BF_KERNEL_BOARD) {
         if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
         if (a->shape.d_model == 512)

@@ -1,0 +1,6 @@
+// Kernel variant "twin256_fp8" of the evaluator (one position per workgroup, e4m3), compiled as its own translation unit.
+#include "bf_board.hip.h"
+
+namespace bf {
+hipError_t launch_twin256_fp8(const KArgs& k, hipStream_t stream) { return board::launch_board<256, false, true, true>(k, stream); }
+}  // namespace bf

@@ -241,19 +241,29 @@ def pack_network(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_v
     return wstream, fparams
 
 
-def pack_network_board(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_value: int):
-    """state_dict -> (board_wstream uint8, board_fparams float32): the int8 network in the order
-    of the one-position-per-workgroup kernel (layout at the end of include/brokefish_hip.h).
+def pack_network_board(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: int, n_value: int,
+                       fmt: str = "int8"):
+    """state_dict -> (board_wstream uint8, board_fparams float32): the network in the order of the
+    one-position-per-workgroup kernels (layout at the end of include/brokefish_hip.h), in the
+    int8 or (256-wide network only) the e4m3 format.
     Wave w owns tiles tw*w .. tw*w+tw-1 of the width; each wave gets its own weight stream and
     its own slice of the side parameters."""
+    if fmt not in ("int8", "e4m3") or (fmt == "e4m3" and d != 256):
+        raise ValueError(f"fmt = {fmt!r} at width {d}: expected 'int8', or 'e4m3' at width 256")
+    fp8 = fmt == "e4m3"
     nt, tw, kc, kcf = d // 32, d // 128, d // 256, f // 256
     cw = 32 * tw
     get = lambda k: sd[k].detach().float().cpu()
     quant = []
     for l in range(n_layers):
         p = f"encoder.layers.{l}."
-        quant.append([quantise_weights_int8(get(p + nm)) for nm in
-                      ("self_attn.in_proj_weight", "self_attn.out_proj.weight", "linear1.weight", "linear2.weight")])
+        mats = [get(p + nm) for nm in
+                ("self_attn.in_proj_weight", "self_attn.out_proj.weight", "linear1.weight", "linear2.weight")]
+        if fp8:   # scales [N/128, K/256]: one k-chunk for the three 256-deep matmuls
+            qs = [quantise_weights_e4m3(m) for m in mats]
+            quant.append([(q, sc[:, 0]) for q, sc in qs[:3]] + [qs[3]])
+        else:
+            quant.append([quantise_weights_int8(m) for m in mats])
     head = np.zeros((128, d), np.float32)
     head[:N_POLICY] = get("policy.weight").numpy()
     head[N_POLICY:N_POLICY + N_PROMO] = get("promo.weight").numpy()
@@ -290,13 +300,19 @@ def pack_network_board(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: in
                       b_qkv[:d][own], b_qkv[d:2 * d][own], b_qkv[2 * d:][own],
                       get(p + "self_attn.out_proj.bias").numpy()[own], sw_a]
             hidden = np.concatenate([np.arange(512 * st + 128 * w, 512 * st + 128 * w + 128) for st in range(f // 512)])
-            wsum = (128 * q_ff2.astype(np.int32).reshape(d, kcf, 256).sum(axis=2)).T[:, own]   # [kcf, cw]
+            if fp8:
+                wsum = np.zeros((kcf, cw), np.int32)      # no unsigned operand in this format
+            else:
+                wsum = (128 * q_ff2.astype(np.int32).reshape(d, kcf, 256).sum(axis=2)).T[:, own]   # [kcf, cw]
             sw_b = np.zeros(32, np.float32)
             for st in range(f // 512):
                 for i in range(4):
                     sw_b[4 * st + i] = s_ff1[(512 * st + 128 * w + 32 * i) // BLOCK_N]
             for i, n in enumerate(tiles):
-                sw_b[16 + i] = s_ff2[(32 * n) // BLOCK_N]
+                if fp8:   # one scale per (own tile, k-chunk)
+                    sw_b[16 + i * kcf:16 + (i + 1) * kcf] = s_ff2[(32 * n) // BLOCK_N]
+                else:
+                    sw_b[16 + i] = s_ff2[(32 * n) // BLOCK_N]
             part_b = [get(p + "norm2.weight").numpy()[own], get(p + "norm2.bias").numpy()[own],
                       get(p + "linear1.bias").numpy()[hidden], get(p + "linear2.bias").numpy()[own],
                       np.ascontiguousarray(wsum, dtype=np.int32).view(np.float32).reshape(-1), sw_b]
@@ -372,8 +388,8 @@ class FusedEncoder:
         if wide and kernel in ("quad", "twin"):
             raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernel "
                                       "(kernel='board' or 'auto') only")
-        if fp8 and kernel in ("board", "twin"):
-            raise NotImplementedError("the one-position-per-workgroup kernels run in int8 only")
+        if fp8 and kernel == "board":
+            raise NotImplementedError("e4m3 runs on the 'twin' and 'quad' kernels")
         if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
             raise ValueError("the evaluator implements pre-norm ReLU layers only")
         self.n_value = int(net.value.weight.shape[0]) if net is not None else 1
@@ -415,8 +431,9 @@ class FusedEncoder:
                 raise RuntimeError("packed blob sizes disagree with the library's layout")
             self.wstream = torch.from_numpy(wstream).to(self.device)
             self.fparams = torch.from_numpy(fparams).to(self.device)
-        if not self.fp8 and kernel != "quad":
-            wstream, fparams = pack_network_board(sd, self.n_layers, self.d_model, self.d_ff, self.n_value)
+        if kernel != "quad":
+            wstream, fparams = pack_network_board(sd, self.n_layers, self.d_model, self.d_ff, self.n_value,
+                                                  fmt="e4m3" if self.fp8 else "int8")
             if wstream.size != self._lib.bf_board_wstream_bytes(C.byref(self._shape)) or \
                     fparams.size != self._lib.bf_board_fparams_floats(C.byref(self._shape)):
                 raise RuntimeError("packed blob sizes disagree with the library's layout (board kernel)")

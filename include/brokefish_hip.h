@@ -43,8 +43,9 @@ enum bf_quant {
  *   TWIN   the BOARD decomposition shaped so that two workgroups share a compute unit (each SIMD
  *          holds two wavefronts that cover each other's waits): the highest throughput
  *          (256-wide network).
- * BOARD and TWIN read the same blobs (board_wstream / board_fparams), int8 only.  For the
- * 256-wide network all three return bit-identical results, so AUTO may pick by batch size. */
+ * BOARD and TWIN read the same blobs (board_wstream / board_fparams); BOARD runs int8, TWIN
+ * int8 and e4m3.  For the 256-wide network all kernels that carry a format return bit-identical
+ * results in it, so AUTO may pick by batch size. */
 enum bf_kernel {
     BF_KERNEL_AUTO = 0,
     BF_KERNEL_QUAD = 1,
@@ -76,8 +77,8 @@ size_t bf_layer_stride_floats(const bf_shape* s); /* stride of one layer inside 
  * feed-forward hidden activations occupy the register file.  Contents are meaningless
  * between launches; launches that may overlap need separate workspaces. */
 size_t bf_workspace_bytes(const bf_shape* s, int64_t n);
-/* The same two blobs in the order of the BOARD and TWIN kernels (int8 only); 0 for an
- * unsupported shape.  Those kernels need no workspace. */
+/* The same two blobs in the order of the BOARD and TWIN kernels (the sizes do not depend on
+ * the format); 0 for an unsupported shape.  Those kernels need no workspace. */
 size_t bf_board_wstream_bytes(const bf_shape* s);
 size_t bf_board_fparams_floats(const bf_shape* s);
 
@@ -138,9 +139,9 @@ typedef struct {
      * to this call); wstream / fparams / workspace may be NULL when QUAD is not to run */
     const uint8_t* board_wstream;
     const float* board_fparams;
-    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs and int8: BOARD for the
+    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: int8 -> BOARD for the
                              * 512-wide network and for n <= bf_board_max_n(), TWIN above;
-                             * otherwise QUAD */
+                             * e4m3 -> TWIN; without them QUAD */
 } bf_eval_args;
 
 /* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */
@@ -217,7 +218,8 @@ const char* bf_profile_phase_name(int i);
  * (own channels, d/4 each) sw_q[TW] sw_k[TW] sw_v[TW] sw_out[TW] (per own tile, padded to 16);
  * part B  ln2_gamma ln2_beta (own) b_ffn1 (own hidden channels: 128 per step) b_ffn2 (own)
  * wsum[d_ff/256][d/4] (int32, own channels) sw_ffn1[4 per step, padded to 16] sw_ffn2[TW]
- * (padded to 16); after the four waves the embedding tables and norm_f as below.
+ * (padded to 16; in the e4m3 format sw_ffn2[TW][d_ff/256], one per own tile and k-chunk, and
+ * wsum all zero); after the four waves the embedding tables and norm_f as below.
  *
  * fparams (fp32 unless noted), per layer at stride bf_layer_stride_floats() (the layer's
  * parameters zero-padded to a multiple of 4 KiB, because a workgroup copies them to LDS

@@ -114,10 +114,30 @@ def test_automatic_choice_switches_kernel_by_batch_size_without_changing_results
     for x, y in zip(big, ref):
         assert torch.equal(x, y)
     fp8 = encoder_impl("hip")(net, fp8=True)
-    assert fp8.kernel_choice(1) == "quad" and fp8.kernel_choice(4096) == "quad"
-    for k in ("board", "twin"):
-        with pytest.raises(NotImplementedError):
-            encoder_impl("hip")(net, fp8=True, kernel=k)
+    assert fp8.kernel_choice(1) == "twin" and fp8.kernel_choice(4096) == "twin"
+    with pytest.raises(NotImplementedError):
+        encoder_impl("hip")(net, fp8=True, kernel="board")
+
+
+def test_e4m3_on_the_throughput_kernel_equals_the_four_per_workgroup_kernel(base):
+    # same quantiser, same MFMA sequence per accumulator, same reduction orders: the same bits
+    # (the e4m3 parity statement against the emulation is in tests/test_parity_fp8_gpu.py)
+    net, sd, boards, quad, co = base
+    twin = encoder_impl("hip")(net, fp8=True, out_dtype=torch.float32, kernel="twin")
+    ref = encoder_impl("hip")(net, fp8=True, out_dtype=torch.float32, kernel="quad")
+    b, c, r, m = positions.random_positions(333, plies=120, seed=23)
+    bd, cd, rd, md = _dev(b, c, r, m)
+    got = [t.clone() for t in twin.forward_masked(bd, cd, rd, md)]
+    want = ref.forward_masked(bd, cd, rd, md)
+    for x, y in zip(got, want):
+        assert torch.equal(x, y)
+    assert torch.isfinite(twin.forward_full(bd, cd, rd)[0]).all()
+    tt = twin.forward_taps(bd[:40], cd[:40], rd[:40])
+    tq = ref.forward_taps(bd[:40], cd[:40], rd[:40])
+    for k in TAPS:
+        assert tt[k].dtype == tq[k].dtype and torch.equal(tt[k].view(torch.uint8), tq[k].view(torch.uint8)), k
+    int8 = boards["twin"].forward_full(bd, cd, rd)[0]
+    assert not torch.equal(int8, twin.forward_full(bd, cd, rd)[0])
 
 
 def test_full_batch_at_4096_on_the_throughput_kernel(base):
