@@ -115,6 +115,9 @@ struct KArgs {
     bf_taps taps;
 };
 
+// Text returned by bf_last_error() on this thread (set by every translation unit of the library).
+void set_error(const char* msg);
+
 // One launcher per separately compiled kernel variant (production, debug taps, phase
 // profile); each sets the dynamic-LDS limit once and launches on `stream`.
 hipError_t launch_prod(const KArgs& k, int grid, hipStream_t stream);

@@ -15,6 +15,8 @@ static int fail(int code, const char* msg) {
     return code;
 }
 
+void bf::set_error(const char* msg) { snprintf(g_err, sizeof(g_err), "%s", msg); }
+
 static bool shape_ok(const bf_shape* s) {   // the four-positions-per-workgroup kernel
     return s && s->d_model == bf::D && s->d_ff == bf::F && s->n_heads == bf::NH && s->n_layers >= 1 &&
            (s->n_value == 1 || s->n_value == 3);

@@ -51,6 +51,14 @@ class _Taps(C.Structure):
                 + [(n, C.c_void_p) for n in _TAP_PTRS])
 
 
+class _ExpandArgs(C.Structure):
+    _fields_ = [("policy", C.c_void_p), ("promo", C.c_void_p), ("value", C.c_void_p), ("mask", C.c_void_p),
+                ("boards", C.c_void_p), ("control", C.c_void_p), ("active", C.c_void_p), ("n", C.c_int64),
+                ("max_edges", C.c_int32), ("logits_fp32", C.c_int32), ("edge_move", C.c_void_p),
+                ("edge_prior", C.c_void_p), ("n_edges", C.c_void_p), ("count", C.c_void_p),
+                ("dropped", C.c_void_p), ("node_value", C.c_void_p)]
+
+
 class _Args(C.Structure):
     _fields_ = [("boards", C.c_void_p), ("control", C.c_void_p), ("rep", C.c_void_p),
                 ("mask", C.c_void_p), ("n", C.c_int64), ("shape", _Shape),
@@ -98,6 +106,8 @@ def load_library():
         L.bf_board_wstream_bytes.argtypes = [C.POINTER(_Shape)]
         L.bf_board_fparams_floats.restype = C.c_size_t
         L.bf_board_fparams_floats.argtypes = [C.POINTER(_Shape)]
+        L.bf_expand.restype = C.c_int
+        L.bf_expand.argtypes = [C.POINTER(_ExpandArgs), C.c_void_p]
         L.bf_board_max_n.restype = C.c_int64
         L.bf_kernel_choice.restype = C.c_int
         L.bf_kernel_choice.argtypes = [C.POINTER(_Args)]
@@ -115,6 +125,61 @@ def int8_q_max():
 def fp8_q_max() -> float:
     """The e4m3 quantisation maximum compiled into the library."""
     return float(load_library().bf_fp8_q_max())
+
+
+def expand_edges(policy, promo, value, mask, boards, control, max_edges: int = 96, active=None, out=None):
+    """The search's expand step on the device, behind the evaluator (docs/reference/search.md:616-636,
+    brokefish/search/torch_impl.py:962-1033): logits + legal-move words -> edges in canonical order.
+
+    ``policy [n,32,64]``, ``promo [n,32,4]`` (fp16 or fp32, as ``forward_full`` returns them),
+    ``value [n]`` fp32, ``mask [n,32]`` int64, ``boards [n,32]`` int16, ``control [n]`` int16, all on
+    the GPU.  Returns a dict: ``edge_move [n,E]`` int16 (slot*64+square | type << 11), ``edge_prior
+    [n,E]`` fp16, ``n_edges [n]`` int32, ``count [n]`` int32 (candidates before truncation to
+    ``max_edges``), ``dropped [n]`` fp32 (prior mass truncated away), ``node_value [n]`` fp16 =
+    (value+1)/2.  ``active`` ([n] bool/uint8) leaves the rows where it is 0 untouched; ``out`` reuses
+    a dict returned earlier.  The launch is asynchronous on the current stream."""
+    n = policy.shape[0]
+    if policy.shape != (n, T, N_POLICY) or promo.shape != (n, T, N_PROMO) or policy.dtype != promo.dtype or \
+            policy.dtype not in (torch.float16, torch.float32):
+        raise ValueError("policy must be [n,32,64] and promo [n,32,4], both fp16 or both fp32")
+    if value.shape != (n,) or value.dtype is not torch.float32:
+        raise ValueError(f"value must be [{n}] float32")
+    if mask.shape != (n, T) or mask.dtype is not torch.int64 or boards.shape != (n, T) or boards.dtype is not torch.int16 \
+            or control.shape != (n,) or control.dtype is not torch.int16:
+        raise ValueError("mask must be [n,32] int64, boards [n,32] int16, control [n] int16")
+    if not 1 <= max_edges <= 255:
+        raise ValueError("max_edges must be in [1, 255] (edge indices are uint8 in the search)")
+    tensors = [policy, promo, value, mask, boards, control] + ([active] if active is not None else [])
+    if any(not t.is_cuda for t in tensors):
+        raise ValueError("all inputs must be on the GPU")
+    dev = policy.device
+    if out is None:
+        out = {"edge_move": torch.zeros(n, max_edges, dtype=torch.int16, device=dev),
+               "edge_prior": torch.zeros(n, max_edges, dtype=torch.float16, device=dev),
+               "n_edges": torch.zeros(n, dtype=torch.int32, device=dev),
+               "count": torch.zeros(n, dtype=torch.int32, device=dev),
+               "dropped": torch.zeros(n, dtype=torch.float32, device=dev),
+               "node_value": torch.zeros(n, dtype=torch.float16, device=dev)}
+    elif out["edge_move"].shape != (n, max_edges):
+        raise ValueError("`out` was made for another n or max_edges")
+    a = _ExpandArgs()
+    keep = [t.contiguous() for t in (policy, promo, value, mask, boards, control)]
+    a.policy, a.promo, a.value, a.mask, a.boards, a.control = [t.data_ptr() for t in keep]
+    if active is not None:
+        act = active.to(torch.uint8).contiguous()
+        if act.shape != (n,):
+            raise ValueError(f"active must be [{n}]")
+        a.active = act.data_ptr()
+    a.n, a.max_edges, a.logits_fp32 = n, max_edges, int(policy.dtype is torch.float32)
+    a.edge_move, a.edge_prior, a.n_edges = out["edge_move"].data_ptr(), out["edge_prior"].data_ptr(), out["n_edges"].data_ptr()
+    a.count, a.dropped, a.node_value = out["count"].data_ptr(), out["dropped"].data_ptr(), out["node_value"].data_ptr()
+    lib = load_library()
+    rc = lib.bf_expand(C.byref(a), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    if rc:
+        raise RuntimeError(f"bf_expand failed ({rc}): {lib.bf_last_error().decode()}")
+    if any(k is not t for k, t in zip(keep, (policy, promo, value, mask, boards, control))) or active is not None:
+        torch.cuda.current_stream(dev).synchronize()     # temporaries made above must outlive the launch
+    return out
 
 
 # --------------------------------------------------------------------------- #
@@ -522,6 +587,14 @@ class FusedEncoder:
         if rc < 0:
             raise RuntimeError(f"bf_kernel_choice failed ({rc}): {self._lib.bf_last_error().decode()}")
         return {1: "quad", 2: "board", 3: "twin"}[rc]
+
+    def forward_expand(self, boards, control, rep, mask, max_edges: int = 96, active=None, out=None):
+        """``forward_full`` followed on the same stream by the search's expand step
+        (:func:`expand_edges`): one evaluator launch, one expansion launch, no host round trip.
+        Returns the edge dict; the logits stay available as ``policy_out`` / ``promo_out`` /
+        ``value_out`` until the next call."""
+        policy, promo, value = self.forward_full(boards, control, rep)
+        return expand_edges(policy, promo, value, mask, boards, control, max_edges, active, out)
 
     def _call(self, args: _Args) -> None:
         rc = self._lib.bf_model_forward(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream))

@@ -185,6 +185,46 @@ int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_t* cycles);
 int bf_profile_phase_count(void);
 const char* bf_profile_phase_name(int i);
 
+/* Edge expansion behind the evaluator: turns the logits of n positions and their legal-move
+ * words into the edges of search nodes, on the device, with no host round trip.  Replaces the
+ * expand step of the reference's search (reference docs/reference/search.md:616-636;
+ * brokefish/search/torch_impl.py:962-1033; device twin csrc/search.cuh:540-798).
+ *
+ * Per position: the set bits of the 32 mask words are enumerated in canonical order (ascending
+ * slot, then square; a move of a live pawn onto the last rank of the side to move -- rank 8 when
+ * control > 0, rank 1 when control < 0 -- gives four edges in the order N B R Q).  An edge's
+ * log-prior is policy[slot][square], plus log_softmax(promo[slot])[type] for a promotion edge.
+ * If there are more than max_edges candidates the max_edges largest are kept (ties by canonical
+ * order; the survivors stay in canonical order).  edge_prior is the softmax over the survivors.
+ *   edge_move  [n, max_edges] int16   slot*64+square | type << 11; 0 beyond n_edges
+ *   edge_prior [n, max_edges] fp16    0 beyond n_edges
+ *   n_edges    [n] int32; count [n] int32 (candidates before truncation, optional);
+ *   dropped    [n] fp32 (prior mass removed by the truncation, optional);
+ *   node_value [n] fp16 = (value + 1) / 2 (optional; needs value).
+ * active (optional, [n] uint8): positions with 0 are left untouched.  policy / promo are the
+ * evaluator's outputs: fp16, or fp32 when logits_fp32 is set; policy may be raw or already
+ * masked (only legal entries are read).  A position with no legal move gets n_edges = 0. */
+typedef struct {
+    const void* policy;
+    const void* promo;
+    const float* value;
+    const uint64_t* mask;
+    const uint16_t* boards;
+    const int16_t* control;
+    const uint8_t* active;
+    int64_t n;
+    int32_t max_edges;      /* 1 .. 255 (the reference's E, 96 by default) */
+    int32_t logits_fp32;
+    int16_t* edge_move;
+    void* edge_prior;
+    int32_t* n_edges;
+    int32_t* count;
+    float* dropped;
+    void* node_value;
+} bf_expand_args;
+
+int bf_expand(const bf_expand_args* args, void* stream);
+
 /* -------------------------------------------------------------------------------------
  * Blob layouts (what the host packer writes; brokefish_amd/hip_impl.py is the packer).
  *
