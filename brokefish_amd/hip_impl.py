@@ -108,6 +108,8 @@ def load_library():
         L.bf_board_fparams_floats.argtypes = [C.POINTER(_Shape)]
         L.bf_expand.restype = C.c_int
         L.bf_expand.argtypes = [C.POINTER(_ExpandArgs), C.c_void_p]
+        L.bf_movegen.restype = C.c_int
+        L.bf_movegen.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.bf_board_max_n.restype = C.c_int64
         L.bf_kernel_choice.restype = C.c_int
         L.bf_kernel_choice.argtypes = [C.POINTER(_Args)]
@@ -125,6 +127,31 @@ def int8_q_max():
 def fp8_q_max() -> float:
     """The e4m3 quantisation maximum compiled into the library."""
     return float(load_library().bf_fp8_q_max())
+
+
+def movegen(boards, control, out=None):
+    """Legal-move words on the device (the reference's ``env.movegen``, docs/reference/spec.md:152-172):
+    ``boards [n,32]`` int16, ``control [n]`` int16 on the GPU -> ``(mask [n,32] int64, in_check [n] bool)``.
+    ``out`` reuses a pair returned earlier.  Asynchronous on the current stream."""
+    n = boards.shape[0]
+    if boards.shape != (n, T) or boards.dtype is not torch.int16 or control.shape != (n,) or control.dtype is not torch.int16:
+        raise ValueError("boards must be [n,32] int16 and control [n] int16")
+    if not boards.is_cuda or not control.is_cuda:
+        raise ValueError("boards and control must be on the GPU")
+    if not boards.is_contiguous() or not control.is_contiguous():
+        raise ValueError("boards and control must be contiguous")
+    if out is None:
+        out = (torch.empty(n, T, dtype=torch.int64, device=boards.device),
+               torch.empty(n, dtype=torch.bool, device=boards.device))
+    mask, chk = out
+    if mask.shape != (n, T) or mask.dtype is not torch.int64 or chk.shape != (n,) or chk.dtype is not torch.bool:
+        raise ValueError("`out` was made for another n")
+    lib = load_library()
+    rc = lib.bf_movegen(boards.data_ptr(), control.data_ptr(), n, mask.data_ptr(), chk.data_ptr(),
+                        C.c_void_p(torch.cuda.current_stream(boards.device).cuda_stream))
+    if rc:
+        raise RuntimeError(f"bf_movegen failed ({rc}): {lib.bf_last_error().decode()}")
+    return mask, chk
 
 
 def expand_edges(policy, promo, value, mask, boards, control, max_edges: int = 96, active=None, out=None):
@@ -588,13 +615,20 @@ class FusedEncoder:
             raise RuntimeError(f"bf_kernel_choice failed ({rc}): {self._lib.bf_last_error().decode()}")
         return {1: "quad", 2: "board", 3: "twin"}[rc]
 
-    def forward_expand(self, boards, control, rep, mask, max_edges: int = 96, active=None, out=None):
+    def forward_expand(self, boards, control, rep, mask=None, max_edges: int = 96, active=None, out=None):
         """``forward_full`` followed on the same stream by the search's expand step
-        (:func:`expand_edges`): one evaluator launch, one expansion launch, no host round trip.
-        Returns the edge dict; the logits stay available as ``policy_out`` / ``promo_out`` /
-        ``value_out`` until the next call."""
+        (:func:`expand_edges`), with the legal-move words generated on the device
+        (:func:`movegen`) when ``mask`` is not given: two or three launches, no host round trip.
+        Returns the edge dict (plus ``mask`` / ``in_check`` when generated here); the logits stay
+        available as ``policy_out`` / ``promo_out`` / ``value_out`` until the next call."""
+        extra = {}
+        if mask is None:
+            mask, chk = movegen(boards, control)
+            extra = {"mask": mask, "in_check": chk}
         policy, promo, value = self.forward_full(boards, control, rep)
-        return expand_edges(policy, promo, value, mask, boards, control, max_edges, active, out)
+        edges = expand_edges(policy, promo, value, mask, boards, control, max_edges, active, out)
+        edges.update(extra)
+        return edges
 
     def _call(self, args: _Args) -> None:
         rc = self._lib.bf_model_forward(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream))

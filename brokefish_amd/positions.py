@@ -65,6 +65,17 @@ def movegen(boards: np.ndarray, control: np.ndarray):
     return mask, chk
 
 
+def step(boards: np.ndarray, control: np.ndarray, move: np.ndarray, promo: np.ndarray):
+    """Apply ``move[i] = slot * 64 + target`` (promotion type ``promo[i]``: 0 N, 1 B, 2 R, 3 Q) to
+    position i; returns new (boards uint16 [n,32], control int16 [n])."""
+    b = np.array(boards, dtype=np.uint16, copy=True)
+    c = np.array(control, dtype=np.int16, copy=True)
+    mv = np.ascontiguousarray(move, dtype=np.int16)
+    pr = np.ascontiguousarray(promo, dtype=np.uint8)
+    lib().bf_chess_step(b.ctypes.data, c.ctypes.data, mv.ctypes.data, pr.ctypes.data, b.shape[0])
+    return b, c
+
+
 def random_positions_np(n: int, plies: int = 120, seed: int = 0, first_game: int = 0,
                         stamp_queen: bool = False):
     """numpy version: boards uint16 [n,32], control int16 [n], rep uint8 [n], mask uint64 [n,32].

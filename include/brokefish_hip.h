@@ -225,6 +225,15 @@ typedef struct {
 
 int bf_expand(const bf_expand_args* args, void* stream);
 
+/* Legal-move words on the device.  Replaces env.movegen of the reference (reference
+ * docs/reference/spec.md:152-172; brokefish/env/torch_impl.py:251-289): for each of n positions
+ * (boards [n,32] uint16, control [n] int16) writes mask [n,32] uint64 -- bit s of word p set iff
+ * slot p may legally move to square s (spec.md:141-143) -- and, if in_check is not NULL, whether
+ * the side to move is in check.  Positions are assumed well formed (spec.md:108-116: both kings
+ * alive in slots 15 and 31).  Asynchronous on `stream`. */
+int bf_movegen(const uint16_t* boards, const int16_t* control, int64_t n, uint64_t* mask,
+               uint8_t* in_check, void* stream);
+
 /* -------------------------------------------------------------------------------------
  * Blob layouts (what the host packer writes; brokefish_amd/hip_impl.py is the packer).
  *
