@@ -101,6 +101,7 @@ struct KArgs {
     const int16_t* control;
     const uint8_t* rep;
     const uint64_t* mask;
+    const uint8_t* active;        // optional [n]: positions with 0 are skipped, their outputs untouched
     int n;
     const uint8_t* wstream;
     const float* fparams;

@@ -131,6 +131,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t = lane & 31, g = lane >> 5;
     const int b = blockIdx.x;
+    if (a.active && !a.active[b]) return;   // a skipped position: the whole workgroup leaves before any barrier
     const int nl_run = a.l1 - a.l0;
 
     uint8_t* const myring = lds + wave * (SLOTS * BLOCK);   // !TWIN

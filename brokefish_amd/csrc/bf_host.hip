@@ -145,7 +145,7 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     if (!board && (!a->workspace || ((uintptr_t)a->workspace & 15) || a->workspace_bytes < bf_workspace_bytes(&a->shape, a->n)))
         return fail(BF_ERR_ARGUMENT, "workspace must be 16-byte aligned and hold bf_workspace_bytes(shape, n) bytes");
     memset(k, 0, sizeof(*k));
-    k->boards = a->boards; k->control = a->control; k->rep = a->rep; k->mask = a->mask;
+    k->boards = a->boards; k->control = a->control; k->rep = a->rep; k->mask = a->mask; k->active = a->active;
     k->n = (int)a->n;
     k->wstream = ws; k->fparams = fp;
     k->policy = a->policy; k->promo = a->promo; k->value = a->value; k->best = a->best_move;

@@ -142,7 +142,8 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t = lane & 31, g = lane >> 5;
     const int board_raw = blockIdx.x * WAVES + wave;
-    const bool valid = board_raw < a.n;
+    // a skipped position keeps its wavefront (the workgroup's barriers need it) but stores nothing
+    const bool valid = board_raw < a.n && !(a.active && !a.active[board_raw < a.n ? board_raw : 0]);
     const int b = valid ? board_raw : a.n - 1;  // idle waves shadow the last board, store nothing
 
     Stream st;

@@ -66,7 +66,8 @@ class _Args(C.Structure):
                 ("policy", C.c_void_p), ("promo", C.c_void_p), ("value", C.c_void_p),
                 ("best_move", C.c_void_p), ("out_fp32", C.c_int32), ("quant", C.c_int32),
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("taps", C.POINTER(_Taps)),
-                ("board_wstream", C.c_void_p), ("board_fparams", C.c_void_p), ("kernel", C.c_int32)]
+                ("board_wstream", C.c_void_p), ("board_fparams", C.c_void_p), ("active", C.c_void_p),
+                ("kernel", C.c_int32)]
 
 
 _lib = None
@@ -581,8 +582,9 @@ class FusedEncoder:
                 raise ValueError(f"{name} must be on the GPU")
         return n
 
-    def _args(self, boards, control, rep, mask, policy, promo, value, best, taps=None) -> _Args:
+    def _args(self, boards, control, rep, mask, policy, promo, value, best, taps=None, active=None) -> _Args:
         a = _Args()
+        a.active = active.data_ptr() if active is not None else None
         a.boards, a.control, a.rep = boards.data_ptr(), control.data_ptr(), rep.data_ptr()
         a.mask = mask.data_ptr() if mask is not None else None
         a.n = boards.shape[0]
@@ -625,7 +627,7 @@ class FusedEncoder:
         if mask is None:
             mask, chk = movegen(boards, control)
             extra = {"mask": mask, "in_check": chk}
-        policy, promo, value = self.forward_full(boards, control, rep)
+        policy, promo, value = self.forward_full(boards, control, rep, active=active)
         edges = expand_edges(policy, promo, value, mask, boards, control, max_edges, active, out)
         edges.update(extra)
         return edges
@@ -675,20 +677,26 @@ class FusedEncoder:
 
     __call__ = forward
 
-    def forward_full(self, boards, control, rep, mask=None):
+    def forward_full(self, boards, control, rep, mask=None, active=None):
         """Boards to ``(policy_logits, promo, value)`` in one launch.
 
         Without ``mask`` the policy is raw, as the reference evaluator returns it.  With
         ``mask`` illegal entries are ``-inf`` and ``self.best_move`` ([n] int32) is the
         masked argmax.  Returns views on internal buffers, which the next call overwrites.
+        ``active`` ([n] uint8 or bool on the GPU, e.g. the search's leaf flags) skips the
+        positions where it is 0: their rows of the output buffers keep what they held.
         """
         self._require_net("forward_full")
         n = self._check_inputs(boards, control, rep, mask)
         self._ensure_full_buffers(n)
         boards, control, rep = boards.contiguous(), control.contiguous(), rep.contiguous()
         mask = mask.contiguous() if mask is not None else None
+        if active is not None:
+            if active.shape != (n,) or active.dtype not in (torch.uint8, torch.bool) or not active.is_cuda:
+                raise ValueError(f"active must be [{n}] uint8 or bool on the GPU")
+            active = active.contiguous().view(torch.uint8)
         self._call(self._args(boards, control, rep, mask, self.policy_out, self.promo_out,
-                              self.value_out, self.best_out))
+                              self.value_out, self.best_out, active=active))
         self.best_move = self.best_out if mask is not None else None
         return self.policy_out, self.promo_out, self.value_out
 

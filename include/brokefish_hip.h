@@ -139,6 +139,12 @@ typedef struct {
      * to this call); wstream / fparams / workspace may be NULL when QUAD is not to run */
     const uint8_t* board_wstream;
     const float* board_fparams;
+    /* optional [n] uint8: positions with 0 are skipped and their outputs left untouched -- the
+     * flat leaf staging of the reference's search (brokefish/search/cuda_impl.py:137-145:
+     * leaf_board / leaf_control / leaf_rep / leaf_flags) evaluated without compaction and without
+     * paying for the leaves that need no evaluation (BOARD / TWIN: the workgroup exits at once;
+     * QUAD: the wavefront runs on, storing nothing) */
+    const uint8_t* active;
     int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: int8 -> BOARD for the
                              * 512-wide network and for n <= bf_board_max_n(), TWIN above;
                              * e4m3 -> TWIN; without them QUAD */

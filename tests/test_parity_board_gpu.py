@@ -140,6 +140,28 @@ def test_e4m3_on_the_throughput_kernel_equals_the_four_per_workgroup_kernel(base
     assert not torch.equal(int8, twin.forward_full(bd, cd, rd)[0])
 
 
+@pytest.mark.parametrize("kernel", ["board", "twin", "quad"])
+def test_skipped_positions_keep_their_output_rows(base, kernel):
+    # the search's flat leaf staging: only flagged leaves are evaluated (reference
+    # brokefish/search/cuda_impl.py:137-145), the others cost nothing and change nothing
+    net, sd, boards, quad, co = base
+    model = quad if kernel == "quad" else boards[kernel]
+    b, c, r, m = positions.random_positions(203, plies=120, seed=24)
+    bd, cd, rd, md = _dev(b, c, r, m)
+    full = [t.clone() for t in model.forward_masked(bd, cd, rd, md)]
+    act = (torch.arange(203) % 3 != 1).cuda()
+    for t in (model.policy_out, model.promo_out, model.value_out, model.best_out):
+        t.fill_(5)
+    p, q, v = model.forward_full(bd, cd, rd, md, active=act)
+    for got, want in zip((p, q, v, model.best_out), full):
+        assert torch.equal(got[act], want[act])
+        assert (got[~act] == 5).all()
+    p2 = model.forward_full(bd, cd, rd, md, active=act.to(torch.uint8))[0]
+    assert torch.equal(p2[act], full[0][act])
+    with pytest.raises(ValueError):
+        model.forward_full(bd, cd, rd, md, active=act[:10])
+
+
 def test_full_batch_at_4096_on_the_throughput_kernel(base):
     net, sd, boards, quad, co = base
     auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
