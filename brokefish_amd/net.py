@@ -72,3 +72,71 @@ class BrokefishNet(nn.Module):
         self.norm_f.weight.copy_(1.0 + 0.2 * torch.randn(self.d_model, generator=g))
         self.norm_f.bias.copy_(0.1 * torch.randn(self.d_model, generator=g))
         return self
+
+
+# --------------------------------------------------------------------------- #
+# checkpoint conventions (reference brokefish/nn/model.py:173-248)
+# --------------------------------------------------------------------------- #
+# Checkpoints are bare state_dicts; what a file was trained with is recovered from the shape of
+# `value.weight` and from optional marker buffers whose absence is the legacy answer.
+
+VALUE_MODE_ID = {"pooled": 1, "prenorm": 2}      # brokefish/nn/model.py:93
+REINJECT_MODE_ID = {"ln1": 1, "both": 2}         # brokefish/nn/model.py:115
+RULE_FEATURES_ID = 1                             # brokefish/nn/model.py:153
+
+
+def n_value_of(state: dict) -> int:
+    """How many value rows a ``state_dict`` was trained with (1: tanh scalar, 3: win/draw/loss)."""
+    w = state.get("value.weight")
+    if w is None:
+        raise KeyError("no `value.weight` in this state_dict, so its value head cannot be sized. "
+                       "Pass the network's weights, not a training checkpoint")
+    return int(w.shape[0])
+
+
+def _mode_of(state: dict, key: str, ids: dict, legacy: str) -> str:
+    if key not in state:
+        return legacy
+    got = int(state[key])
+    for name, i in ids.items():
+        if i == got:
+            return name
+    raise ValueError(f"unknown {key} {got} in this state_dict; this build knows {ids}")
+
+
+def value_head_of(state: dict) -> str:
+    """Which value head a ``state_dict`` was written with; no marker means the king select."""
+    return _mode_of(state, "value_mode", VALUE_MODE_ID, "king")
+
+
+def reinject_of(state: dict) -> str:
+    """Which per-layer input re-injection a ``state_dict`` was written with; no marker: none."""
+    return _mode_of(state, "reinject_mode", REINJECT_MODE_ID, "none")
+
+
+def rule_features_of(state: dict) -> bool:
+    """Whether a ``state_dict`` carries the rule-derived piece inputs; no marker: it does not."""
+    if "rule_features_mode" not in state:
+        return False
+    got = int(state["rule_features_mode"])
+    if got != RULE_FEATURES_ID:
+        raise ValueError(f"unknown rule_features_mode {got} in this state_dict; this build knows {RULE_FEATURES_ID}")
+    return True
+
+
+def net_for_state(state: dict, **kw) -> BrokefishNet:
+    """An empty net shaped to hold ``state`` (load into it).  Width, depth and feed-forward width
+    are read off the tensors unless given; a head or input variant this library does not carry
+    raises ``NotImplementedError`` from the constructor."""
+    n_layers = 0
+    while f"encoder.layers.{n_layers}.linear1.weight" in state:
+        n_layers += 1
+    if not n_layers or "emb_square.weight" not in state:
+        raise KeyError("not a network state_dict: no encoder layers / embedding tables in it")
+    d_model = int(state["emb_square.weight"].shape[1])
+    kw.setdefault("d_model", d_model)
+    kw.setdefault("n_layers", n_layers)
+    kw.setdefault("n_heads", d_model // 32)
+    kw.setdefault("d_ff", int(state["encoder.layers.0.linear1.weight"].shape[0]))
+    return BrokefishNet(n_value=n_value_of(state), value_head=value_head_of(state),
+                        reinject=reinject_of(state), rule_features=rule_features_of(state), **kw)

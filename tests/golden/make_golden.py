@@ -16,7 +16,7 @@ What it records, and why these need the reference itself rather than a closed fo
   under ``emulated_forward(..., QuantConfig(fmt="int8"))`` (quant.py:498-506) on a net
   whose weights are filled by the formula in :func:`fill_state_dict` (independent of any
   RNG stream) and on eight build-defined positions, plus the layer-0 inputs of the first
-  patched matmul.
+  patched matmul, and ``weight_fingerprint`` (brokefish/train/sync.py:34-49) of that net.
 
 * the e4m3 twins (second file): ``fp8_linear`` (quant.py:360-397), ``quantise_activations``
   (:172-188) and ``quantise_weights_bytes`` (:208-224) on the same inputs with the shipped
@@ -158,6 +158,13 @@ def main() -> int:
         out[f"int8_policy_{tag}"], out[f"int8_promo_{tag}"], out[f"int8_value_{tag}"] = p8.numpy(), q8.numpy(), v8.numpy()
         if n_value == 1:
             out["ln1_layer0"] = captured[0][:2].numpy()        # input of the first patched matmul, boards 0-1
+            # the module file alone: its package's __init__ needs a logging library that is not installed
+            import importlib.util
+            spec = importlib.util.spec_from_file_location("ref_sync", os.path.join(REFERENCE, "brokefish", "train", "sync.py"))
+            ref_sync = importlib.util.module_from_spec(spec)
+            sys.modules["ref_sync"] = ref_sync                 # its dataclass looks its module up by name
+            spec.loader.exec_module(ref_sync)
+            out["weight_fingerprint_nv1"] = np.array(ref_sync.weight_fingerprint(net), np.float64)
     out["torch_version"] = np.array(torch.__version__)
     path = os.path.join(HERE, "reference_vectors.npz")
     np.savez_compressed(path, **out)

@@ -1,0 +1,100 @@
+"""``brokefish_amd.sync``: the weight-snapshot bookkeeping of the reference's training loop
+(brokefish/train/sync.py:34-106) for the HIP evaluator.
+
+``weight_fingerprint`` is pinned by the value the reference's own function returned for the
+formula-weight network (tests/golden/make_golden.py) and by its defining properties: it moves
+when a value moves and when two values swap places.
+"""
+import pytest
+import torch
+
+import make_golden as mg
+from brokefish_amd import sync
+from brokefish_amd.net import BrokefishNet
+
+
+def _golden_net():
+    torch.manual_seed(0)
+    net = BrokefishNet(n_value=1).eval()
+    net.load_state_dict(mg.fill_state_dict(net.state_dict()))
+    return net
+
+
+def test_fingerprint_equals_the_references(golden):
+    assert sync.weight_fingerprint(_golden_net()) == float(golden["weight_fingerprint_nv1"])
+
+
+def test_fingerprint_sees_a_changed_value_and_a_permutation():
+    net = _golden_net()
+    f0 = sync.weight_fingerprint(net)
+    with torch.no_grad():
+        w = net.encoder.layers[3].linear1.weight
+        a, b = w[5, 7].item(), w[5, 8].item()
+        assert a != b
+        w[5, 7], w[5, 8] = b, a                      # same multiset of values, other order
+    f1 = sync.weight_fingerprint(net)
+    with torch.no_grad():
+        w[5, 7], w[5, 8] = a, b
+        net.norm_f.bias[0] += 1e-3
+    f2 = sync.weight_fingerprint(net)
+    assert f1 != f0 and f2 != f0 and f2 != f1
+
+
+def test_pack_argument_rules_do_not_need_a_gpu():
+    net = BrokefishNet(n_layers=1)
+    with pytest.raises(ValueError):
+        sync.PackedWeights.pack(net, 0, fp8=True, int8=True)
+    with pytest.raises(ValueError):
+        sync.PackedWeights.pack(net, 0, impl="cuda", int8=True)
+
+
+@pytest.mark.gpu
+def test_a_stale_snapshot_is_refused():
+    from brokefish_amd import positions
+    net = _golden_net()
+    packed = sync.PackedWeights.pack(net, weight_gen=3, int8=True)
+    packed.assert_current(net, 3)
+    b, c, r, _ = positions.random_positions(8, plies=40, seed=1)
+    policy, promo, value = packed.evaluate()(b.cuda(), c.cuda(), r.cuda())
+    assert policy.dtype is torch.float16 and policy.shape == (8, 32, 64) and value.dtype is torch.float32
+    before = policy.clone()
+    with pytest.raises(AssertionError, match="generation 3"):
+        packed.assert_current(net, 4)
+    with torch.no_grad():
+        net.policy.weight[0, 0] += 0.5                # a gradient step outside the loop's accounting
+    with pytest.raises(AssertionError, match="fingerprint"):
+        packed.assert_current(net, 3)
+    # the snapshot still evaluates the OLD weights: that is exactly why the check exists
+    assert torch.equal(packed.evaluate()(b.cuda(), c.cuda(), r.cuda())[0], before)
+    fresh = sync.PackedWeights.pack(net, weight_gen=4, fp8=True)
+    fresh.assert_current(net, 4)
+    assert fresh.encoder.fp8 and not torch.equal(fresh.evaluate()(b.cuda(), c.cuda(), r.cuda())[0], before)
+
+
+def test_checkpoint_conventions_size_a_net_from_a_bare_state_dict():
+    # reference brokefish/nn/model.py:173-248: the value width from value.weight, the variants from
+    # optional marker buffers whose absence is the legacy answer
+    from brokefish_amd import net as bn
+    for d, heads, layers, nv in ((256, 8, 8, 1), (256, 8, 3, 3), (512, 16, 2, 1)):
+        src = BrokefishNet(d_model=d, n_heads=heads, d_ff=4 * d, n_layers=layers, n_value=nv)
+        state = src.state_dict()
+        assert bn.n_value_of(state) == nv and bn.value_head_of(state) == "king"
+        assert bn.reinject_of(state) == "none" and bn.rule_features_of(state) is False
+        dst = bn.net_for_state(state)
+        dst.load_state_dict(state, strict=True)
+        assert (dst.d_model, dst.n_layers, dst.n_value) == (d, layers, nv)
+        assert sync.weight_fingerprint(dst) == sync.weight_fingerprint(src)
+    state = BrokefishNet(n_layers=1).state_dict()
+    with pytest.raises(KeyError):
+        bn.n_value_of({k: v for k, v in state.items() if k != "value.weight"})
+    for key, val, fn in (("value_mode", 1, "pooled"), ("value_mode", 2, "prenorm")):
+        marked = dict(state, **{key: torch.tensor(val)})
+        assert bn.value_head_of(marked) == fn
+        with pytest.raises(NotImplementedError):
+            bn.net_for_state(marked)                       # recognised, and loudly not carried
+    assert bn.reinject_of(dict(state, reinject_mode=torch.tensor(2))) == "both"
+    assert bn.rule_features_of(dict(state, rule_features_mode=torch.tensor(1))) is True
+    with pytest.raises(ValueError):
+        bn.value_head_of(dict(state, value_mode=torch.tensor(9)))
+    with pytest.raises(ValueError):
+        bn.rule_features_of(dict(state, rule_features_mode=torch.tensor(2)))
