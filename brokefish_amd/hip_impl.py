@@ -738,6 +738,20 @@ class FusedEncoder:
 
     # -- debug taps (the counterpart of the reference's forward_stage) ------------
 
+    def forward_stage(self, boards, control, rep, stage: int):
+        """Activations at an intermediate stage, as reference nn/cuda_impl.py:512-531:
+        stage 9 is the embedding sum alone, stage 8 the output of ``norm_f``; both come back as
+        [n, 32, d] float32.  Stages 1-7 name points inside the reference's own kernel (its
+        staging buffers between phases) and have no counterpart here: ``forward_taps`` exposes
+        this kernel's intermediates (operand bytes, accumulators, residual stream) instead.
+        """
+        self._require_net("forward_stage")
+        if stage not in (8, 9):
+            raise NotImplementedError(f"stage {stage}: only 9 (embeddings) and 8 (after norm_f) exist; "
+                                      "see forward_taps for the per-layer intermediates")
+        key = "embed" if stage == 9 else "normed"
+        return self.forward_taps(boards, control, rep, want=[key])[key]
+
     def forward_taps(self, boards, control, rep, mask=None, x_in=None, layer_begin: int = 0,
                      layer_end: Optional[int] = None, want=None):
         """Run with intermediate outputs.  Returns a dict of fresh fp32-output tensors:

@@ -61,6 +61,11 @@ def test_bit_exact_against_the_c_checker_with_every_tap(nets, key):
     want = co.forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy(), taps=True)
     for k in TAPS_INT + TAPS_F32 + ["policy", "promo", "value", "best"]:
         assert _bits_equal(got[k], want[k]), k
+    # the reference's stage numbers that exist outside its kernel: 9 = embeddings, 8 = norm_f output
+    assert _bits_equal(model.forward_stage(*_dev(b, c, r), 9), want["embed"])
+    assert _bits_equal(model.forward_stage(*_dev(b, c, r), 8), want["normed"])
+    with pytest.raises(NotImplementedError):
+        model.forward_stage(*_dev(b, c, r), 3)
     # the accumulators really are the exact integer product of the kernel's own operand bytes
     q, _ = co.qweight("ff2", 3)
     a = got["qa_ff2"][:, 3].cpu().numpy().astype(np.int64)                 # [n,32,1024] unsigned
