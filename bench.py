@@ -7,7 +7,8 @@ in HBM and outputs preallocated before the timed region.  Prints ONE JSON line.
 Extra objects in the line:
   roofline      dense-int8 MFMA roofline of the evaluator kernel: algorithmic int8 ops per
                 launch (402,653,184 per evaluation x batch) over the kernel's average duration
-                measured with HIP events on the launch stream.
+                measured with HIP events on the launch stream; `measured_mfma_rate` is the rate
+                a register-resident loop of the same MFMA instruction reaches on this GPU (TOP/s).
   cpu_baseline  the CPU port of the same forward (oracle/emulated.py, PyTorch on the host
                 cores) timed on a bounded sample of the same workload.
 """
@@ -134,6 +135,10 @@ def main() -> int:
                      "traffic": None if fp8 else MEASURED_TRAFFIC_BYTES.get((a.shape, model.kernel_choice(a.batch), a.batch)),
                      "kernel_ms": kern_ms, "ops_per_launch": ops_per_eval * a.batch},
     }
+    # the matrix pipe's measured ceiling for the instruction the kernel uses (register-resident
+    # MFMA chains, no memory traffic), next to the datasheet peak that `frac` is quoted against
+    from brokefish_amd.hip_impl import mfma_rate
+    line["roofline"]["measured_mfma_rate"] = mfma_rate(a.quant)
     if a.sweep:
         # the batch-size sweep of the small-batch latency regime: same net, same generator
         pts = []

@@ -19,7 +19,7 @@ INCLUDE = os.path.join(ROOT, "include")
 HIP_LIB = os.path.join(HERE, "libbrokefish_hip.so")
 CHESSGEN_LIB = os.path.join(HERE, "libbf_chessgen.so")
 
-HIP_SOURCES = ["bf_host.hip", "bf_expand.hip", "bf_movegen.hip", "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip",
+HIP_SOURCES = ["bf_host.hip", "bf_expand.hip", "bf_movegen.hip", "bf_probe.hip", "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip",
                "bf_variant_prod_fp8.hip", "bf_variant_taps_fp8.hip",
                "bf_variant_board256.hip", "bf_variant_board256_taps.hip",
                "bf_variant_board512.hip", "bf_variant_board512_taps.hip",

@@ -1,0 +1,107 @@
+// Matrix-pipe rate probe: a register-resident loop of independent MFMA chains with no memory
+// traffic inside the loop, so a measured ceiling stands next to the datasheet peak the
+// evaluator's roofline is quoted against.  Same method as the reference's own ceiling
+// measurement (reference docs/ledger/perf.md:616-642: raw mma in a register-resident loop with
+// eight independent accumulators).
+//
+// Every wavefront keeps four independent 32x32 accumulators and issues them round-robin; two
+// wavefronts per SIMD give eight chains in flight per matrix pipe.  Operands are read once from
+// `scratch` (so nothing folds to a constant) and the accumulators are stored back only under a
+// condition the data never meets, which keeps the loop alive without a store in it.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+
+#include "bf_args.h"
+
+namespace {
+
+typedef long v2l __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int CHAINS = 4;
+constexpr int PROBE_THREADS = 256;
+
+template <bool FP8>
+__global__ __launch_bounds__(PROBE_THREADS) void mfma_loop(int* scratch, int iters) {
+    const int lane = threadIdx.x & 63;
+    const v4i a = *reinterpret_cast<const v4i*>(scratch + 4 * lane);
+    const v4i b = *reinterpret_cast<const v4i*>(scratch + 256 + 4 * lane);
+    int fold = 0;
+    if constexpr (FP8) {
+        const v2l al = __builtin_bit_cast(v2l, a), bl = __builtin_bit_cast(v2l, b);
+        v16f acc[CHAINS];
+#pragma unroll
+        for (int c = 0; c < CHAINS; c++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[c][i] = 0.0f;
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int c = 0; c < CHAINS; c++) {
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[0], bl[0], acc[c], 0, 0, 0);
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[1], bl[1], acc[c], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CHAINS; c++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) fold ^= __float_as_int(acc[c][i]);
+    } else {
+        v16i acc[CHAINS];
+#pragma unroll
+        for (int c = 0; c < CHAINS; c++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[c][i] = 0;
+        for (int it = 0; it < iters; it++) {
+#pragma unroll
+            for (int c = 0; c < CHAINS; c++)
+                acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[c], 0, 0, 0);
+        }
+#pragma unroll
+        for (int c = 0; c < CHAINS; c++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) fold ^= acc[c][i];
+    }
+    // zero operands give zero accumulators: this store never happens on the probe's own input
+    if (fold == 0x5bd1e995) scratch[512 + lane] = fold;
+}
+
+}  // namespace
+
+extern "C" double bf_mfma_rate(int quant, int* scratch, int iters, int reps, void* stream) {
+    auto fail = [](int code, const char* msg) {
+        bf::set_error(msg);
+        return (double)code;
+    };
+    if (quant != BF_QUANT_INT8 && quant != BF_QUANT_E4M3) return fail(BF_ERR_ARGUMENT, "quant must be BF_QUANT_INT8 or BF_QUANT_E4M3");
+    if (!scratch || ((uintptr_t)scratch & 15)) return fail(BF_ERR_ARGUMENT, "scratch must be a 16-byte aligned device buffer of 4096 zero bytes");
+    if (iters < 1 || iters > (1 << 24) || reps < 1 || reps > 1000) return fail(BF_ERR_ARGUMENT, "iters must be in [1, 2^24] and reps in [1, 1000]");
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+        return fail(BF_ERR_LAUNCH, "cannot read the compute-unit count");
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(2 * cus), block(PROBE_THREADS);     // two wavefronts per SIMD
+    auto go = [&]() {
+        if (quant == BF_QUANT_E4M3) hipLaunchKernelGGL(mfma_loop<true>, grid, block, 0, s, scratch, iters);
+        else hipLaunchKernelGGL(mfma_loop<false>, grid, block, 0, s, scratch, iters);
+    };
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    go();                                               // warm-up: code load and clock ramp
+    (void)hipEventRecord(e0, s);
+    for (int r = 0; r < reps; r++) go();
+    (void)hipEventRecord(e1, s);
+    const hipError_t e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    const hipError_t le = hipGetLastError();
+    if (e != hipSuccess || le != hipSuccess) return fail(BF_ERR_LAUNCH, hipGetErrorString(e != hipSuccess ? e : le));
+    // 2*32*32*32 operations per int8 instruction; the e4m3 chain step is two 32x32x16 instructions
+    const double ops = 65536.0 * CHAINS * (double)iters * (PROBE_THREADS / 64) * grid.x * reps;
+    return ops / ((double)ms * 1e-3) / 1e12;
+}

@@ -114,6 +114,8 @@ def load_library():
         L.bf_board_max_n.restype = C.c_int64
         L.bf_kernel_choice.restype = C.c_int
         L.bf_kernel_choice.argtypes = [C.POINTER(_Args)]
+        L.bf_mfma_rate.restype = C.c_double
+        L.bf_mfma_rate.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         _lib = L
     return _lib
 
@@ -128,6 +130,20 @@ def int8_q_max():
 def fp8_q_max() -> float:
     """The e4m3 quantisation maximum compiled into the library."""
     return float(load_library().bf_fp8_q_max())
+
+
+def mfma_rate(fmt: str = "int8", iters: int = 20000, reps: int = 5, device="cuda") -> float:
+    """Measured rate of the matrix pipe in TOP/s for the MFMA instruction of ``fmt`` ("int8" or
+    "e4m3"): register-resident independent chains on every compute unit, no memory traffic in
+    the loop (the method of reference docs/ledger/perf.md:616-642).  Synchronises."""
+    L = load_library()
+    scratch = torch.zeros(1024, dtype=torch.int32, device=device)
+    with torch.cuda.device(scratch.device):
+        rate = L.bf_mfma_rate({"int8": 0, "e4m3": 1}[fmt], scratch.data_ptr(), iters, reps,
+                              torch.cuda.current_stream().cuda_stream)
+    if rate < 0:
+        raise RuntimeError(f"bf_mfma_rate: {L.bf_last_error().decode()}")
+    return float(rate)
 
 
 def movegen(boards, control, out=None):

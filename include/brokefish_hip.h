@@ -179,6 +179,17 @@ const char* bf_last_error(void);
  * (reference csrc/encoder.cu:1886-1903) at whole-kernel granularity. */
 double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int iters);
 
+/* Measured rate of the matrix pipe, in TOP/s: a register-resident loop of independent
+ * 32x32 MFMA chains (v_mfma_i32_32x32x32_i8 for BF_QUANT_INT8, v_mfma_f32_32x32x16_fp8_fp8 for
+ * BF_QUANT_E4M3), two wavefronts per SIMD on every compute unit, no memory traffic inside the
+ * loop; `iters` chain steps per wavefront, `reps` timed launches after one warm-up launch.
+ * `scratch` is a 16-byte aligned DEVICE buffer of 4096 zero bytes.  Returns a negative
+ * bf_status on error.  Synchronises the stream.  The evaluator's roofline is quoted against
+ * the datasheet peak; this number says how much of that peak the instruction the kernels use
+ * reaches on the installed part.  Follows the reference's own ceiling measurement (reference
+ * docs/ledger/perf.md:616-642). */
+double bf_mfma_rate(int quant, int* scratch, int iters, int reps, void* stream);
+
 /* In-kernel phase accounting, the counterpart of the reference's profile hooks
  * (reference csrc/encoder.cu:1083-1177 and :1886-1903: set_profile / read_profile /
  * profile_phases).  bf_profile_phases runs a separately compiled build of the evaluator

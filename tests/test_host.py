@@ -57,6 +57,9 @@ def test_null_arguments_are_rejected_without_a_launch():
     a.shape = hip_impl._Shape(384, 8, 12, 1536, 1, 1e-5)
     assert lib.bf_model_forward(ctypes.byref(a), None) == -2
     assert lib.bf_model_forward(None, None) == -1
+    # the matrix-pipe probe rejects a missing buffer and a bad format before touching a device
+    assert lib.bf_mfma_rate(0, None, 10, 1, None) == -1.0
+    assert lib.bf_mfma_rate(7, ctypes.c_void_p(4096), 10, 1, None) == -1.0
 
 
 def test_kernel_choice_follows_shape_blobs_and_batch_size():

@@ -241,3 +241,12 @@ def test_stress_network_win_draw_loss_head_and_full_batch_properties():
     assert torch.isneginf(p[~legal]).all() and torch.isfinite(p[legal]).all() and (v.abs() <= 1).all()
     has = legal.reshape(n, -1).any(1)
     assert torch.gather(legal.reshape(n, -1)[has], 1, best[has].long()[:, None]).all()
+
+
+def test_matrix_pipe_probe_reports_a_plausible_rate():
+    # a register-resident MFMA loop cannot beat the datasheet peak (5.0 POP/s dense int8 / fp8)
+    # and, on a healthy part, reaches most of it; the evaluator's own rate must lie below it
+    from brokefish_amd.hip_impl import mfma_rate
+    for fmt in ("int8", "e4m3"):
+        rate = mfma_rate(fmt, iters=5000, reps=3)
+        assert 1000.0 < rate < 5500.0, (fmt, rate)
