@@ -139,8 +139,11 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     const float* fp = board ? a->board_fparams : a->fparams;
     if (((uintptr_t)ws & 15) || ((uintptr_t)fp & 15))
         return fail(BF_ERR_ARGUMENT, "the parameter blobs must be 16-byte aligned");
-    if (((uintptr_t)a->policy & 15) || ((uintptr_t)a->promo & 7) || ((uintptr_t)a->boards & 1))
+    if (((uintptr_t)a->policy & 15) || ((uintptr_t)a->promo & 7))
         return fail(BF_ERR_ARGUMENT, "policy must be 16-byte and promo 8-byte aligned");
+    if (((uintptr_t)a->boards & 1) || ((uintptr_t)a->control & 1) || ((uintptr_t)a->value & 3) ||
+        ((uintptr_t)a->mask & 7) || ((uintptr_t)a->best_move & 3))
+        return fail(BF_ERR_ARGUMENT, "boards/control/value/mask/best_move must be aligned to their element size");
     if (a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
     if (!board && (!a->workspace || ((uintptr_t)a->workspace & 15) || a->workspace_bytes < bf_workspace_bytes(&a->shape, a->n)))
         return fail(BF_ERR_ARGUMENT, "workspace must be 16-byte aligned and hold bf_workspace_bytes(shape, n) bytes");
@@ -230,8 +233,11 @@ extern "C" double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int 
     if (iters < 1 || warmup < 0) return fail(BF_ERR_ARGUMENT, "iters must be >= 1 and warmup >= 0");
     hipStream_t s = (hipStream_t)stream;
     hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+    if (hipEventCreate(&e0) != hipSuccess) return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    if (hipEventCreate(&e1) != hipSuccess) {
+        (void)hipEventDestroy(e0);
         return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    }
     for (int i = 0; i < warmup && !rc; i++) rc = launch(args, k, kind, s);
     (void)hipEventRecord(e0, s);
     for (int i = 0; i < iters && !rc; i++) rc = launch(args, k, kind, s);

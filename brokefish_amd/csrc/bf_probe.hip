@@ -89,7 +89,11 @@ extern "C" double bf_mfma_rate(int quant, int* scratch, int iters, int reps, voi
         else hipLaunchKernelGGL(mfma_loop<false>, grid, block, 0, s, scratch, iters);
     };
     hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    if (hipEventCreate(&e0) != hipSuccess) return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    if (hipEventCreate(&e1) != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    }
     go();                                               // warm-up: code load and clock ramp
     (void)hipEventRecord(e0, s);
     for (int r = 0; r < reps; r++) go();

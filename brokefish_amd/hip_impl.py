@@ -623,7 +623,7 @@ class FusedEncoder:
         return a
 
     def kernel_choice(self, n: int) -> str:
-        """Which kernel a call with ``n`` positions runs ("quad" or "board")."""
+        """Which kernel a call with ``n`` positions runs ("quad", "board" or "twin")."""
         a = _Args()
         a.n, a.shape, a.quant, a.kernel = n, self._shape, (1 if self.fp8 else 0), self.KERNELS[self.kernel]
         a.wstream = a.fparams = 16 if self.wstream is not None else None        # only tested for NULL
@@ -735,15 +735,20 @@ class FusedEncoder:
         return ms
 
     def profile_phases(self, boards, control, rep, mask=None) -> Dict[str, float]:
-        """Shader-clock cycles per phase, averaged over the wavefronts of one launch (the
-        counterpart of the reference's read_profile / profile_phases)."""
+        """Shader-clock cycles per phase, averaged over the wavefronts of one launch of the
+        four-positions-per-workgroup kernel's profiling build (the counterpart of the
+        reference's read_profile / profile_phases).  The outputs it writes are the normal ones."""
         n = self._check_inputs(boards, control, rep, mask)
+        if self.wstream is None or self.fp8:
+            raise NotImplementedError("the phase profile is a build of the four-positions-per-workgroup int8 "
+                                      "kernel: construct with int8=True and kernel='auto' or 'quad'")
         self._ensure_full_buffers(n)
         k = self._lib.bf_profile_phase_count()
         cyc = torch.zeros(k, dtype=torch.int64, device=self.device)
         args = self._args(boards.contiguous(), control.contiguous(), rep.contiguous(),
                           mask.contiguous() if mask is not None else None,
                           self.policy_out, self.promo_out, self.value_out, self.best_out)
+        args.kernel = self.KERNELS["quad"]
         rc = self._lib.bf_profile_phases(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
                                          C.c_void_p(cyc.data_ptr()))
         if rc:
