@@ -181,6 +181,22 @@ def test_full_batch_at_4096_on_the_throughput_kernel(base):
     assert torch.isneginf(p[~legal]).all() and torch.isfinite(p[legal]).all() and (v.abs() <= 1).all()
 
 
+def test_largest_batch_of_the_sweep_is_independent_of_batch_composition(base):
+    # 65536 positions (the top of the batch sweep): 2048 distinct positions repeated 32 times in a
+    # shuffled order must each come back with the bits the 2048-position launch gave them
+    net, sd, boards, quad, co = base
+    model = encoder_impl("hip")(net, int8=True)              # fp16 logits, the search's contract
+    b, c, r, m = positions.random_positions(2048, plies=120, seed=31)
+    small = [t.clone() for t in model.forward_masked(*_dev(b, c, r, m))]
+    g = torch.Generator().manual_seed(7)
+    order = torch.cat([torch.randperm(2048, generator=g) for _ in range(32)])
+    assert model.kernel_choice(65536) == "twin"
+    big = model.forward_masked(*_dev(b[order], c[order], r[order], m[order]))
+    od = order.cuda()
+    for got, want in zip(big, small):
+        assert got.shape[0] == 65536 and torch.equal(got, want[od])
+
+
 def test_stress_network_bit_exact_against_the_c_checker_with_every_tap(stress):
     net, sd, model, co = stress
     assert model.kernel_choice(16384) == "board" and model.wstream is None
