@@ -221,8 +221,10 @@ def expand_edges(policy, promo, value, mask, boards, control, max_edges: int = 9
     rc = lib.bf_expand(C.byref(a), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
     if rc:
         raise RuntimeError(f"bf_expand failed ({rc}): {lib.bf_last_error().decode()}")
-    if any(k is not t for k, t in zip(keep, (policy, promo, value, mask, boards, control))) or active is not None:
-        torch.cuda.current_stream(dev).synchronize()     # temporaries made above must outlive the launch
+    # Temporaries made above (contiguous copies, the uint8 view of `active`) were allocated on the
+    # current stream, where the launch is queued: the allocator hands their memory out again only
+    # to work that this stream runs after the kernel, so no host wait is needed (and none would
+    # be legal while a graph is being captured).
     return out
 
 
