@@ -164,8 +164,9 @@ def movegen(boards, control, out=None):
     if mask.shape != (n, T) or mask.dtype is not torch.int64 or chk.shape != (n,) or chk.dtype is not torch.bool:
         raise ValueError("`out` was made for another n")
     lib = load_library()
-    rc = lib.bf_movegen(boards.data_ptr(), control.data_ptr(), n, mask.data_ptr(), chk.data_ptr(),
-                        C.c_void_p(torch.cuda.current_stream(boards.device).cuda_stream))
+    with torch.cuda.device(boards.device):       # the launch goes to the current device
+        rc = lib.bf_movegen(boards.data_ptr(), control.data_ptr(), n, mask.data_ptr(), chk.data_ptr(),
+                            C.c_void_p(torch.cuda.current_stream(boards.device).cuda_stream))
     if rc:
         raise RuntimeError(f"bf_movegen failed ({rc}): {lib.bf_last_error().decode()}")
     return mask, chk
@@ -218,7 +219,8 @@ def expand_edges(policy, promo, value, mask, boards, control, max_edges: int = 9
     a.edge_move, a.edge_prior, a.n_edges = out["edge_move"].data_ptr(), out["edge_prior"].data_ptr(), out["n_edges"].data_ptr()
     a.count, a.dropped, a.node_value = out["count"].data_ptr(), out["dropped"].data_ptr(), out["node_value"].data_ptr()
     lib = load_library()
-    rc = lib.bf_expand(C.byref(a), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
+    with torch.cuda.device(dev):
+        rc = lib.bf_expand(C.byref(a), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream))
     if rc:
         raise RuntimeError(f"bf_expand failed ({rc}): {lib.bf_last_error().decode()}")
     # Temporaries made above (contiguous copies, the uint8 view of `active`) were allocated on the
@@ -601,6 +603,9 @@ class FusedEncoder:
         return n
 
     def _args(self, boards, control, rep, mask, policy, promo, value, best, taps=None, active=None) -> _Args:
+        for name, t in (("boards", boards), ("control", control), ("rep", rep), ("mask", mask), ("active", active)):
+            if t is not None and t.device != self.device:
+                raise ValueError(f"{name} is on {t.device}, the evaluator's weights are on {self.device}")
         a = _Args()
         a.active = active.data_ptr() if active is not None else None
         a.boards, a.control, a.rep = boards.data_ptr(), control.data_ptr(), rep.data_ptr()
@@ -651,7 +656,8 @@ class FusedEncoder:
         return edges
 
     def _call(self, args: _Args) -> None:
-        rc = self._lib.bf_model_forward(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream))
+        with torch.cuda.device(self.device):     # the launch goes to the current device
+            rc = self._lib.bf_model_forward(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream))
         if rc:
             raise RuntimeError(f"bf_model_forward failed ({rc}): {self._lib.bf_last_error().decode()}")
 
@@ -730,8 +736,9 @@ class FusedEncoder:
         args = self._args(boards.contiguous(), control.contiguous(), rep.contiguous(),
                           mask.contiguous() if mask is not None else None,
                           self.policy_out, self.promo_out, self.value_out, self.best_out)
-        ms = self._lib.bf_time_kernel_ms(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
-                                         warmup, iters)
+        with torch.cuda.device(self.device):
+            ms = self._lib.bf_time_kernel_ms(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
+                                             warmup, iters)
         if ms < 0:
             raise RuntimeError(f"bf_time_kernel_ms failed ({ms}): {self._lib.bf_last_error().decode()}")
         return ms
@@ -751,8 +758,9 @@ class FusedEncoder:
                           mask.contiguous() if mask is not None else None,
                           self.policy_out, self.promo_out, self.value_out, self.best_out)
         args.kernel = self.KERNELS["quad"]
-        rc = self._lib.bf_profile_phases(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
-                                         C.c_void_p(cyc.data_ptr()))
+        with torch.cuda.device(self.device):
+            rc = self._lib.bf_profile_phases(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
+                                             C.c_void_p(cyc.data_ptr()))
         if rc:
             raise RuntimeError(f"bf_profile_phases failed ({rc}): {self._lib.bf_last_error().decode()}")
         torch.cuda.current_stream(self.device).synchronize()
