@@ -87,7 +87,7 @@ __device__ __forceinline__ void dma(const float* src, float* dst, int nfloats, i
                                          (__attribute__((address_space(3))) void*)(d + full * FRAG), 16, 0, 0);
 }
 
-// one 16-byte fragment step of a block product: a 32-deep int8 MFMA, or two 16-deep e4m3 MFMAs
+// one 16-byte fragment step of a block product: a 32-deep int8 MFMA, or two 16-deep e4m3 steps
 template <bool SWAP>
 __device__ __forceinline__ v16i frag_mma(const v4i& w, const v4i& act, const v16i& acc) {
     return SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act, w, acc, 0, 0, 0)
@@ -97,9 +97,7 @@ template <bool SWAP>
 __device__ __forceinline__ v16f frag_mma(const v4i& w, const v4i& act, v16f acc) {
     const v2l wl = __builtin_bit_cast(v2l, w), al = __builtin_bit_cast(v2l, act);
 #pragma unroll
-    for (int h = 0; h < 2; h++)
-        acc = SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[h], wl[h], acc, 0, 0, 0)
-                   : __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(wl[h], al[h], acc, 0, 0, 0);
+    for (int h = 0; h < 2; h++) acc = e4m3_step<SWAP>(wl[h], al[h], acc);
     return acc;
 }
 

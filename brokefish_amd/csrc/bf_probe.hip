@@ -17,7 +17,7 @@
 
 namespace {
 
-typedef long v2l __attribute__((ext_vector_type(2)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -32,7 +32,8 @@ __global__ __launch_bounds__(PROBE_THREADS) void mfma_loop(int* scratch, int ite
     const v4i b = *reinterpret_cast<const v4i*>(scratch + 256 + 4 * lane);
     int fold = 0;
     if constexpr (FP8) {
-        const v2l al = __builtin_bit_cast(v2l, a), bl = __builtin_bit_cast(v2l, b);
+        // the e4m3 kernels feed their operands, widened exactly, to the fp16 instruction
+        const v8h ah = __builtin_bit_cast(v8h, a), bh = __builtin_bit_cast(v8h, b);
         v16f acc[CHAINS];
 #pragma unroll
         for (int c = 0; c < CHAINS; c++)
@@ -41,8 +42,8 @@ __global__ __launch_bounds__(PROBE_THREADS) void mfma_loop(int* scratch, int ite
         for (int it = 0; it < iters; it++) {
 #pragma unroll
             for (int c = 0; c < CHAINS; c++) {
-                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[0], bl[0], acc[c], 0, 0, 0);
-                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(al[1], bl[1], acc[c], 0, 0, 0);
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, acc[c], 0, 0, 0);
+                acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bh, ah, acc[c], 0, 0, 0);
             }
         }
 #pragma unroll
@@ -105,7 +106,7 @@ extern "C" double bf_mfma_rate(int quant, int* scratch, int iters, int reps, voi
     (void)hipEventDestroy(e1);
     const hipError_t le = hipGetLastError();
     if (e != hipSuccess || le != hipSuccess) return fail(BF_ERR_LAUNCH, hipGetErrorString(e != hipSuccess ? e : le));
-    // 2*32*32*32 operations per int8 instruction; the e4m3 chain step is two 32x32x16 instructions
+    // 2*32*32*32 operations per int8 instruction; the e4m3 chain step is two 32x32x16 fp16 instructions
     const double ops = 65536.0 * CHAINS * (double)iters * (PROBE_THREADS / 64) * grid.x * reps;
     return ops / ((double)ms * 1e-3) / 1e12;
 }

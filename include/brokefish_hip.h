@@ -29,6 +29,12 @@ enum bf_status {
     BF_ERR_DEVICE = -4      /* not a gfx950 device */
 };
 
+/* Operand format of the four weight matmuls of every layer.
+ *   INT8  exact int32 accumulators; every number of the forward is reproducible bit for bit.
+ *   E4M3  OCP e4m3 operands.  Products and sums run on the fp16 matrix instruction, fed with the
+ *         operand bytes widened exactly, so a k-tile's accumulator is the exact product to fp32
+ *         rounding (the fp8 matrix instructions of gfx950 keep about 16 bits below the largest
+ *         addend and are not used). */
 enum bf_quant {
     BF_QUANT_INT8 = 0,
     BF_QUANT_E4M3 = 1
@@ -180,8 +186,8 @@ const char* bf_last_error(void);
 double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int iters);
 
 /* Measured rate of the matrix pipe, in TOP/s: a register-resident loop of independent
- * 32x32 MFMA chains (v_mfma_i32_32x32x32_i8 for BF_QUANT_INT8, v_mfma_f32_32x32x16_fp8_fp8 for
- * BF_QUANT_E4M3), two wavefronts per SIMD on every compute unit, no memory traffic inside the
+ * 32x32 MFMA chains (v_mfma_i32_32x32x32_i8 for BF_QUANT_INT8; v_mfma_f32_32x32x16_f16 for
+ * BF_QUANT_E4M3, whose operands the kernels widen exactly to fp16), two wavefronts per SIMD on every compute unit, no memory traffic inside the
  * loop; `iters` chain steps per wavefront, `reps` timed launches after one warm-up launch.
  * `scratch` is a 16-byte aligned DEVICE buffer of 4096 zero bytes.  Returns a negative
  * bf_status on error.  Synchronises the stream.  The evaluator's roofline is quoted against

@@ -34,6 +34,7 @@ The two agree to rounding noise, which ``tests/test_oracle.py`` asserts.
 """
 from __future__ import annotations
 
+import contextlib
 import math
 from typing import Dict, Optional
 
@@ -153,6 +154,23 @@ def quantise_weights_e4m3(w: torch.Tensor, q_max: float = Q_MAX_E4M3, tile_k: in
     return _to_e4m3(blocks / s).view(n, k), s.reshape(n // block_n, k // tile_k)
 
 
+# How the product inside one k-tile is summed: False = torch's fp32 matmul (the reference's
+# call, summation order left to the library), True = exact sum rounded once to fp32 (float64
+# holds every partial sum of 256 e4m3 products exactly).  Both are fp32 realisations of the same
+# formula; tests use the second to show what a change of summation order alone does.
+TILE_SUM_EXACT = False
+
+
+@contextlib.contextmanager
+def exact_tile_sums():
+    global TILE_SUM_EXACT
+    old, TILE_SUM_EXACT = TILE_SUM_EXACT, True
+    try:
+        yield
+    finally:
+        TILE_SUM_EXACT = old
+
+
 def fp8_linear(x, w, bias, taps: Optional[dict] = None, name: str = "", q_max: float = Q_MAX_E4M3,
                tile_k: int = ROW_K, block_n: int = BLOCK_N):
     """``F.linear`` with both operands e4m3: the product inside one k-tile in fp32, one
@@ -167,7 +185,10 @@ def fp8_linear(x, w, bias, taps: Optional[dict] = None, name: str = "", q_max: f
     out = torch.zeros((m, n), dtype=torch.float32)
     accs = []
     for t, lo in enumerate(range(0, k, tile_k)):
-        part = aq[:, lo:lo + tile_k] @ wq[:, lo:lo + tile_k].T
+        if TILE_SUM_EXACT:
+            part = (aq[:, lo:lo + tile_k].double() @ wq[:, lo:lo + tile_k].double().T).float()
+        else:
+            part = aq[:, lo:lo + tile_k] @ wq[:, lo:lo + tile_k].T
         if taps is not None:
             accs.append(part.clone())
         part = part * sa[:, t:t + 1]

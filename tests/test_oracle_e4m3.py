@@ -167,6 +167,30 @@ def test_golden_forward_e4m3_functional_route(golden, golden8):
     assert np.abs(got[2].numpy() - golden8["e4m3_value_nv1"]).max() < 2e-2
 
 
+def test_free_running_sensitivity_of_e4m3_is_a_property_of_the_algorithm():
+    # The same torch code with the k-tile products summed exactly (float64, rounded once)
+    # instead of in the library's fp32 order: operands differ only where a quotient sits within
+    # fp32 rounding of an e4m3 tie, yet one such flip is 6 % of the element and moves a board's
+    # logits by ~0.1.  So "logits within 2e-2" holds board by board only for boards without a
+    # flip, for ANY two realisations of the formula that do not share a summation order; this is
+    # the spread a kernel's free-running comparison has to be read against.
+    from brokefish_amd import positions
+    torch.manual_seed(0)
+    net = BrokefishNet().eval()
+    net.randomise_layers_(seed=3)
+    sd = {k: v.detach() for k, v in net.state_dict().items()}
+    b, c, r, _ = positions.random_positions(64, plies=120, seed=11, stamp_queen=True)
+    with torch.no_grad():
+        lib = emulated.forward(sd, b, c, r, mode="e4m3")
+        with emulated.exact_tile_sums():
+            exact = emulated.forward(sd, b, c, r, mode="e4m3")
+        assert not emulated.TILE_SUM_EXACT
+    per_board = (lib[0] - exact[0]).abs().reshape(64, -1).amax(1)
+    assert per_board.median() < 1e-4                      # most boards: no flip, fp32 noise only
+    assert 0.5 < (per_board <= 2e-2).float().mean() < 1.0  # some boards do flip ...
+    assert 2e-2 < per_board.max() < 0.3                    # ... and then move by about 0.1
+
+
 def test_teacher_forcing_entry_points_compose():
     # running layers [0,3) then [3,8) from the recorded residual stream is the whole forward
     sd, b, c, r = _golden_net()
