@@ -30,6 +30,7 @@ PEAK_FP16_OPS = 2.5e15                # dense fp16 MFMA: the e4m3 format's produ
 # (calibrated on a 1 GiB copy), by (network shape, kernel, batch).
 MEASURED_TRAFFIC_BYTES = {("base", "twin", 4096): 1.00e9, ("base", "quad", 4096): 3.07e9,
                           ("base", "board", 256): 5.5e7, ("stress", "board", 16384): 2.66e10}
+MEASURED_TRAFFIC_BYTES_E4M3 = {("base", "twin", 4096): 0.97e9}
 
 
 def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0, mode: str = "int8"):
@@ -134,7 +135,8 @@ def main() -> int:
                                "fp16 logits out, seed-0 random-init weights"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak / 1e12, "unit": "TFLOP/s" if fp8 else "TOP/s",
                      "frac": achieved / (peak / 1e12),
-                     "traffic": None if fp8 else MEASURED_TRAFFIC_BYTES.get((a.shape, model.kernel_choice(a.batch), a.batch)),
+                     "traffic": (MEASURED_TRAFFIC_BYTES_E4M3 if fp8 else MEASURED_TRAFFIC_BYTES).get(
+                         (a.shape, model.kernel_choice(a.batch), a.batch)),
                      "kernel_ms": kern_ms, "ops_per_launch": ops_per_eval * a.batch},
     }
     # the matrix pipe's measured ceiling for the instruction the kernel uses (register-resident
