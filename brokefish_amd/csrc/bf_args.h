@@ -126,9 +126,11 @@ hipError_t launch_taps(const KArgs& k, int grid, hipStream_t stream);
 hipError_t launch_prof(const KArgs& k, int grid, hipStream_t stream);
 hipError_t launch_prod_fp8(const KArgs& k, int grid, hipStream_t stream);
 hipError_t launch_taps_fp8(const KArgs& k, int grid, hipStream_t stream);
-// one position per workgroup (grid = n), int8, for the 256- and the 512-wide network
+// one position per workgroup (grid = n), for the 256- (int8, e4m3) and the 512-wide network (int8)
 hipError_t launch_board256(const KArgs& k, hipStream_t stream);
 hipError_t launch_board256_taps(const KArgs& k, hipStream_t stream);
+hipError_t launch_board256_fp8(const KArgs& k, hipStream_t stream);
+hipError_t launch_board256_fp8_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_board512(const KArgs& k, hipStream_t stream);
 hipError_t launch_board512_taps(const KArgs& k, hipStream_t stream);
 // the same with two workgroups per compute unit (256-wide network)

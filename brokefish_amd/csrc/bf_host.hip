@@ -100,15 +100,15 @@ static int choose_kernel(const bf_eval_args* a) {
         return fail(BF_ERR_ARGUMENT, "quant must be BF_QUANT_INT8 or BF_QUANT_E4M3");
     const bool have_quad = a->wstream && a->fparams, have_board = a->board_wstream && a->board_fparams;
     const bool quad_can = shape_ok(&a->shape) && have_quad;
-    // the board blobs are packed for one format; BOARD runs int8, TWIN both
-    const bool board_can = have_board && a->quant == BF_QUANT_INT8;
+    // the board blobs are packed for one format; the 512-wide network runs int8 only
+    const bool board_can = have_board && (a->quant == BF_QUANT_INT8 || shape_ok(&a->shape));
     const bool twin_can = have_board && shape_ok(&a->shape);
     switch (a->kernel) {
     case BF_KERNEL_QUAD:
         if (!quad_can) return fail(BF_ERR_UNSUPPORTED, "the four-positions-per-workgroup kernel needs the 256-wide network and wstream/fparams");
         return BF_KERNEL_QUAD;
     case BF_KERNEL_BOARD:
-        if (!board_can) return fail(BF_ERR_UNSUPPORTED, "the one-position-per-workgroup kernel needs board_wstream/board_fparams and the int8 format");
+        if (!board_can) return fail(BF_ERR_UNSUPPORTED, "the one-position-per-workgroup kernel needs board_wstream/board_fparams (512-wide network: the int8 format)");
         return BF_KERNEL_BOARD;
     case BF_KERNEL_TWIN:
         if (!twin_can)
@@ -116,7 +116,6 @@ static int choose_kernel(const bf_eval_args* a) {
         return BF_KERNEL_TWIN;
     case BF_KERNEL_AUTO:
         if (board_can) return (twin_can && a->n > kBoardMaxN) ? BF_KERNEL_TWIN : BF_KERNEL_BOARD;
-        if (twin_can) return BF_KERNEL_TWIN;      // e4m3
         if (quad_can) return BF_KERNEL_QUAD;
         return fail(BF_ERR_ARGUMENT, shape512(&a->shape)
                         ? "the 512-wide network runs on the one-position-per-workgroup kernel: int8, board_wstream/board_fparams required"
@@ -181,6 +180,8 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream
         if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
         if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_board512_taps(k, stream) : bf::launch_board512(k, stream);
+        else if (a->quant == BF_QUANT_E4M3)
+            e = a->taps ? bf::launch_board256_fp8_taps(k, stream) : bf::launch_board256_fp8(k, stream);
         else
             e = a->taps ? bf::launch_board256_taps(k, stream) : bf::launch_board256(k, stream);
     } else if (a->quant == BF_QUANT_E4M3)

@@ -501,8 +501,6 @@ class FusedEncoder:
         if wide and kernel in ("quad", "twin"):
             raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernel "
                                       "(kernel='board' or 'auto') only")
-        if fp8 and kernel == "board":
-            raise NotImplementedError("e4m3 runs on the 'twin' and 'quad' kernels")
         if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
             raise ValueError("the evaluator implements pre-norm ReLU layers only")
         self.n_value = int(net.value.weight.shape[0]) if net is not None else 1

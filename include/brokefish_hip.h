@@ -42,16 +42,17 @@ enum bf_quant {
 
 /* Three kernels compute the same function.
  *   QUAD   four positions per workgroup, one wavefront each, weights shared through LDS; carries
- *          the e4m3 format and the phase profile (256-wide network).
+ *          the phase profile (256-wide network, int8 and e4m3).
  *   BOARD  one position per workgroup, the four wavefronts split the model width; one workgroup
  *          per compute unit: the lowest latency per position (launches that cannot fill the GPU)
  *          and the only kernel the 512-wide network fits.
  *   TWIN   the BOARD decomposition shaped so that two workgroups share a compute unit (each SIMD
  *          holds two wavefronts that cover each other's waits): the highest throughput
  *          (256-wide network).
- * BOARD and TWIN read the same blobs (board_wstream / board_fparams); BOARD runs int8, TWIN
- * int8 and e4m3.  For the 256-wide network all kernels that carry a format return bit-identical
- * results in it, so AUTO may pick by batch size. */
+ * BOARD and TWIN read the same blobs (board_wstream / board_fparams).  The 256-wide network runs
+ * in int8 and e4m3 on all three, the 512-wide network in int8 on BOARD.  For the 256-wide network
+ * the three kernels return bit-identical results in either format, so AUTO may pick by batch
+ * size. */
 enum bf_kernel {
     BF_KERNEL_AUTO = 0,
     BF_KERNEL_QUAD = 1,
@@ -65,7 +66,7 @@ enum bf_kernel {
 #define BF_POLICY 64
 #define BF_PROMO 4
 
-/* Network shape.  Supported: d_model 256, n_heads 8, d_ff 1024 (all kernels; e4m3 on QUAD)
+/* Network shape.  Supported: d_model 256, n_heads 8, d_ff 1024 (all kernels, int8 and e4m3)
  * and d_model 512, n_heads 16, d_ff 2048 (BOARD kernel, int8); head width 32, any
  * n_layers >= 1, n_value 1 (tanh scalar) or 3 (loss/draw/win classes). */
 typedef struct {
@@ -151,9 +152,9 @@ typedef struct {
      * paying for the leaves that need no evaluation (BOARD / TWIN: the workgroup exits at once;
      * QUAD: the wavefront runs on, storing nothing) */
     const uint8_t* active;
-    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: int8 -> BOARD for the
-                             * 512-wide network and for n <= bf_board_max_n(), TWIN above;
-                             * e4m3 -> TWIN; without them QUAD */
+    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: BOARD for the 512-wide
+                             * network and for n <= bf_board_max_n(), TWIN above; without
+                             * them QUAD */
 } bf_eval_args;
 
 /* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */
