@@ -221,7 +221,8 @@ extern "C" int bf_movegen(const uint16_t* boards, const int16_t* control, int64_
     };
     if (n < 1 || n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
     if (!boards || !control || !mask) return fail(BF_ERR_ARGUMENT, "boards/control/mask must not be NULL");
-    if (((uintptr_t)boards & 1) || ((uintptr_t)mask & 7)) return fail(BF_ERR_ARGUMENT, "boards must be 2-byte and mask 8-byte aligned");
+    if (((uintptr_t)boards & 1) || ((uintptr_t)control & 1) || ((uintptr_t)mask & 7))
+        return fail(BF_ERR_ARGUMENT, "boards and control must be 2-byte and mask 8-byte aligned");
     hipLaunchKernelGGL(movegen_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, (hipStream_t)stream, boards, control,
                        (int)n, reinterpret_cast<u64*>(mask), in_check);
     const hipError_t e = hipGetLastError();
