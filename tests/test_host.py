@@ -31,6 +31,23 @@ def test_library_loads_and_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} is declared in include/brokefish_hip.h but not exported"
 
 
+def test_header_is_plain_c_and_a_c_client_links_and_gets_statuses(tmp_path):
+    # a C99 program (no C++, no torch, no Python) built against the header and the library:
+    # every argument error must come back as a status before any device is touched
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    exe = tmp_path / "abi_check"
+    lib_dir = os.path.dirname(_build.HIP_LIB)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                    os.path.join(ROOT, "tests", "abi", "abi_check.c"), "-o", str(exe), "-L", lib_dir,
+                    "-lbrokefish_hip", f"-Wl,-rpath,{lib_dir}"], check=True, capture_output=True, text=True)
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
+    assert run.stdout.startswith("abi ok")
+
+
 def test_constants_agree_between_host_and_library():
     # the counterpart of the reference's Python<->CUDA constant pin (tests/test_quant.py:233-269)
     assert hip_impl.int8_q_max() == (hip_impl.Q_MAX_S8, hip_impl.Q_MAX_U8) == (127.0, 255.0)
