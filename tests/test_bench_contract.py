@@ -1,0 +1,40 @@
+"""The benchmark's command-line contract: one JSON line with the agreed keys, and a refusal of
+more than one GPU.  The GPU leg runs the real thing briefly; the refusal needs no GPU."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"],
+                         capture_output=True, text=True, timeout=120)
+    assert run.returncode != 0 and "one GPU" in run.stderr and run.stdout.strip() == ""
+
+
+@pytest.mark.gpu
+def test_one_json_line_with_roofline_and_cpu_baseline():
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "5", "--warmup", "2", "--cpu-batch", "16"],
+                         capture_output=True, text=True, timeout=280)
+    assert run.returncode == 0, run.stderr[-2000:]
+    lines = [l for l in run.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    assert d["metric"] == "network evals/sec at batch 4096 int8 on 1 MI355X" and d["unit"] == "evals/s"
+    assert d["n_gpus"] == 1 and d["steps"] == 5 and d["warmup"] == 2 and d["higher_is_better"] is True
+    assert d["dtype"] == "int8" and d["data"] == "synthetic" and d["vs_baseline"] is None and d["scaling"] == "weak"
+    assert set(d["config"]) == {"workload"} and "batch 4096" in d["config"]["workload"] and "kernel twin" in d["config"]["workload"]
+    assert abs(d["value"] - 4096 / (d["ms_per_step"] * 1e-3)) < 1e-6 * d["value"]
+    r = d["roofline"]
+    assert r["bound"] == "mfma" and r["unit"] == "TOP/s" and r["peak"] == 5000.0
+    assert abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-12
+    assert abs(r["achieved"] - r["ops_per_launch"] / (r["kernel_ms"] * 1e-3) / 1e12) < 1e-6 * r["achieved"]
+    assert r["ops_per_launch"] == 4096 * 402_653_184 and r["traffic"] > 0
+    assert 0.5 * r["peak"] < r["measured_mfma_rate"] < 1.1 * r["peak"]
+    assert d["value"] > 1.0e6          # a sanity bound, far below what the kernel measures (2.1-2.2 M)
+    c = d["cpu_baseline"]
+    assert c["kind"] == "port" and c["unit"] == "evals/s" and c["cores"] >= 1 and c["value"] > 0 and "batch 16" in c["sample"]
