@@ -40,22 +40,30 @@
 #ifndef BF_TWIN_OCC
 #define BF_TWIN_OCC 2
 #endif
+// Eight-wavefront form: one workgroup per compute unit leaves each wave 256 registers of which the
+// kernel needs fewer, and a launch that small is bound by the latency of the weight stream, not
+// by its bandwidth: more half-blocks in flight.
+#ifndef BF_OCTO_SETS
+#define BF_OCTO_SETS 6
+#endif
 
 namespace bf {
 namespace board {
 
 extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
-template <int DM, bool TWIN>
+template <int DM, bool TWIN, bool OCTO = false>
 struct Cfg : Layout<DM> {
     typedef Layout<DM> L;
+    static constexpr int NW = OCTO ? 8 : 4;   // wavefronts per position
     static constexpr int RING_BYTES = TWIN ? 0 : 4 * L::SLOTS * BLOCK;
     static constexpr int XCH_OFF = RING_BYTES;
-    static constexpr int HID_OFF = XCH_OFF + 3 * FRAG;
+    static constexpr int HID_OFF = XCH_OFF + 3 * (NW / 4) * FRAG;
     static constexpr int ACT_OFF = HID_OFF + 16 * FRAG;
     static constexpr int PAR_OFF = ACT_OFF + L::NT * FRAG;
-    static constexpr int LDS_BYTES = PAR_OFF + 4 * L::PW_FLOATS * 4;
-    static_assert(LDS_BYTES <= (TWIN ? 160 / BF_TWIN_OCC : 160) * 1024, "LDS budget: one or two workgroups per compute unit");
+    static constexpr int LDS_BYTES = PAR_OFF + NW * L::PW_FLOATS * 4;
+    static_assert(!OCTO || TWIN, "eight wavefronts per position take their weights straight to registers");
+    static_assert(LDS_BYTES <= (TWIN && !OCTO ? 160 / BF_TWIN_OCC : 160) * 1024, "LDS budget: one or two workgroups per compute unit");
     static_assert(L::NT * 4 * FRAG <= LDS_BYTES - HID_OFF, "normalised stream overlay");
     static_assert(L::BPW % L::SLOTS == 0, "ring slot of a block must not depend on the layer");
     static_assert((2 * L::BPW) % BF_TWIN_SETS == 0, "register set of a half-block must not depend on the layer");
@@ -115,18 +123,43 @@ __device__ __forceinline__ float chunk_sum(const ACC (&acc)[KC], int i, const fl
     }
 }
 
-template <int DM, bool TAPS, bool TWIN, bool FP8>
-__global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(const KArgs a) {
-    typedef Cfg<DM, TWIN> C;
+// Position of a wave's n-th weight block of a layer inside its quarter's stream: a + sub * b.
+// With four wavefronts per position a wave consumes its quarter's stream in order (a = n).  With
+// eight, the two wavefronts of a quarter (sub = 0, 1) each take half of the quarter's tiles in
+// every matmul, so a wave's blocks are every other group of the same stream.
+struct BlockAt { int a, b; };
+template <int KC, int TW, int SUB>
+__host__ __device__ constexpr BlockAt block_at(int n) {
+    constexpr int TWW = TW / SUB, HT = 4 / SUB;
+    constexpr int NQ = 3 * KC * TWW, NO = KC * TWW, SW_ = HT * KC + 2 * TWW;
+    if (n < NQ) return {3 * KC * (n / (3 * KC)) + n % (3 * KC), 3 * KC * TWW};
+    if (n < NQ + NO) return {3 * KC * TW + KC * ((n - NQ) / KC) + (n - NQ) % KC, KC * TWW};
+    const int m = n - NQ - NO, st = m / SW_, r = m % SW_, base = 4 * KC * TW + st * (4 * KC + 2 * TW);
+    if (r < HT * KC) return {base + KC * (r / KC) + r % KC, KC * HT};
+    return {base + 4 * KC + ((r - HT * KC) / TWW) * TW + (r - HT * KC) % TWW, TWW};
+}
+
+template <int DM, bool TAPS, bool TWIN, bool FP8, bool OCTO = false>
+__global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TWIN_OCC : 1) void board_kernel(const KArgs a) {
+    typedef Cfg<DM, TWIN, OCTO> C;
     typedef typename Acc<FP8>::type acc_t;
     static_assert(!FP8 || DM == 256, "e4m3: one k-chunk per matmul of the width (fp32 sums over the chunks of ffn2 only)");
     constexpr int D = C::D, F = C::F, NT = C::NT, TW = C::TW, CW = C::CW, KC = C::KC, KCF = C::KCF;
     constexpr int STEPS = C::STEPS, BPW = C::BPW, HB = C::HB, SLOTS = C::SLOTS, WPC = 4 / KC;
+    constexpr int NW = C::NW, SUB = NW / 4;   // wavefronts per position; wavefronts sharing a quarter of the width
+    constexpr int TWW = TW / SUB;             // tiles of the width a wave owns
+    constexpr int HT = 4 / SUB;               // hidden tiles a wave computes per feed-forward step
+    constexpr int NB = BPW / SUB;             // weight blocks a wave consumes per layer
+    constexpr int NSETS = OCTO ? BF_OCTO_SETS : BF_TWIN_SETS;   // register sets of the prefetch: NSETS - 1 half-blocks in flight
+    static_assert(TW % SUB == 0 && (2 * NB) % NSETS == 0, "tiles and register sets must split evenly");
+    constexpr int XS = NW * 64;               // floats of one exchange slot
     constexpr int HALF = BLOCK / 2;   // four fragments: the unit of the register prefetch (TWIN)
-    constexpr int NSETS = BF_TWIN_SETS;   // register sets of the prefetch: NSETS - 1 half-blocks in flight
     constexpr int VM_AHEAD = TAPS ? 0 : (SLOTS - 1) * 8;   // ring loads that may stay in flight at a ring wait
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = OCTO ? (wave & 3) : wave;   // the quarter of the width this wave works in
+    const int sub = OCTO ? (wave >> 2) : 0;   // which of the quarter's waves it is
+    const int t0 = TWW * sub, h0 = HT * sub;  // its first tile of the quarter, its first hidden tile of a step
     const int t = lane & 31, g = lane >> 5;
     const int b = blockIdx.x;
     if (a.active && !a.active[b]) return;   // a skipped position: the whole workgroup leaves before any barrier
@@ -136,12 +169,12 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     float* const xch = reinterpret_cast<float*>(lds + C::XCH_OFF);
     uint8_t* const hid = lds + C::HID_OFF;
     uint8_t* const act = lds + C::ACT_OFF;
-    float* const pA = reinterpret_cast<float*>(lds + C::PAR_OFF) + wave * C::PW_FLOATS;
+    float* const pA = reinterpret_cast<float*>(lds + C::PAR_OFF) + wave * C::PW_FLOATS;   // every wave keeps its own copy
     float* const pB = pA + C::A_FLOATS;
-    // this wave's weight stream, from the first layer that runs; block `seq` in consumption order
+    // the quarter's weight stream, from the first layer that runs; block `seq` in the quarter's order
     const uint8_t* const wsrc =
-        a.wstream + ((size_t)wave * ((size_t)a.n_layers * BPW + HB + 1) + (size_t)a.l0 * BPW) * BLOCK + lane * 16;
-    const float* const wpar = a.fparams + (size_t)wave * a.n_layers * C::PW_FLOATS;   // this wave's [layer][PW]
+        a.wstream + ((size_t)q * ((size_t)a.n_layers * BPW + HB + 1) + (size_t)a.l0 * BPW) * BLOCK + lane * 16;
+    const float* const wpar = a.fparams + (size_t)q * a.n_layers * C::PW_FLOATS;   // the quarter's [layer][PW]
     const float* const gp = a.fparams + (size_t)4 * a.n_layers * C::PW_FLOATS;       // tables, final norm
 
     // TWIN: half-block `hseq` of this wave's stream (consumption order) into register set `set`
@@ -150,6 +183,13 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
         const uint8_t* src = wsrc + (size_t)hseq * HALF;
 #pragma unroll
         for (int s = 0; s < 4; s++) frt[set][s] = *reinterpret_cast<const v4i*>(src + s * FRAG);
+    };
+    // the wave's hh-th half-block of the layer whose stream starts at block `base` (hh may run into
+    // the following layer, whose stream starts at block `next`) into its register set
+    auto fetch_half = [&](int hh, int base, int next) {
+        const int n = hh / 2;
+        const BlockAt at = block_at<KC, TW, SUB>(n % NB);
+        load_half(2 * ((n < NB ? base : next) + at.a + sub * at.b) + hh % 2, hh % NSETS);
     };
     // !TWIN: block `seq` into ring slot `slot`; a slot into the fragment registers
     v4i fr[8];
@@ -165,35 +205,51 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
 #pragma unroll
         for (int s = 0; s < 8; s++) fr[s] = *reinterpret_cast<const v4i*>(&myring[slot * BLOCK + s * FRAG + lane * 16]);
     };
-    // sum of a per-lane value over the four waves, in wave order
-    auto xsum = [&](float v, int slot) -> float {
-        xch[slot * 256 + wave * 64 + lane] = v;
-        lds_barrier();
-        const float* p = xch + slot * 256 + lane;
-        return ((p[0] + p[64]) + p[128]) + p[192];
+    // Row sum over the width: `chain(start)` adds this wave's values to `start` one by one; a
+    // quarter's values form one chain (with eight waves the quarter's second wave continues the
+    // first one's), and the four quarter sums are added in order.
+    // Four waves: one exchange slot per call site (`slot`), so that a fast wave's next partial
+    // cannot overwrite what a slow wave still reads.  Eight waves: slots 0 and 1 serve every call;
+    // the two barriers of a call separate its traffic from the previous call's.
+    auto xsum = [&](auto&& chain, int slot) -> float {
+        if constexpr (!OCTO) {
+            xch[slot * XS + wave * 64 + lane] = chain(0.0f);
+            lds_barrier();
+            const float* p = xch + slot * XS + lane;
+            return ((p[0] + p[64]) + p[128]) + p[192];
+        } else {
+            if (sub == 0) xch[q * 64 + lane] = chain(0.0f);
+            lds_barrier();
+            if (sub == 1) xch[XS + q * 64 + lane] = chain(xch[q * 64 + lane]);
+            lds_barrier();
+            const float* p = xch + XS + lane;
+            return ((p[0] + p[64]) + p[128]) + p[192];
+        }
     };
     // LayerNorm of this wave's channels; gamma / beta point at this wave's slice
-    auto layernorm = [&](const float (&x)[TW][16], const float* gamma, const float* beta, float (&y)[TW][16]) {
-        float s = 0.0f;
+    auto layernorm = [&](const float (&x)[TWW][16], const float* gamma, const float* beta, float (&y)[TWW][16]) {
+        const float s = xsum([&](float acc) {
 #pragma unroll
-        for (int i = 0; i < TW; i++)
+            for (int i = 0; i < TWW; i++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) s = s + x[i][r];
-        s = xsum(s, 0);
+                for (int r = 0; r < 16; r++) acc = acc + x[i][r];
+            return acc;
+        }, 0);
         const float mean = (s + partner(s, g)) * (1.0f / D);
-        float v = 0.0f;
+        const float v = xsum([&](float acc) {
 #pragma unroll
-        for (int i = 0; i < TW; i++)
+            for (int i = 0; i < TWW; i++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float d = x[i][r] - mean;
-                v = __builtin_fmaf(d, d, v);
-            }
-        v = xsum(v, 1);
+                for (int r = 0; r < 16; r++) {
+                    const float d = x[i][r] - mean;
+                    acc = __builtin_fmaf(d, d, acc);
+                }
+            return acc;
+        }, 1);
         const float var = (v + partner(v, g)) * (1.0f / D);
         const float rstd = 1.0f / __builtin_sqrtf(var + a.eps);
 #pragma unroll
-        for (int i = 0; i < TW; i++)
+        for (int i = 0; i < TWW; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const v4f ga = ldg4(gamma + 32 * i + 8 * j + 4 * g);
@@ -207,45 +263,47 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     };
     // signed quantiser of a row spread over the four waves: per 256-wide chunk one scale; this
     // wave's bytes go to the activation buffer, every wave then reads the whole row back
-    auto quant_exchange = [&](const float (&y)[TW][16], float (&sa)[KC], v4i (&q)[NT], int8_t* tap, size_t tap_row) {
+    auto quant_exchange = [&](const float (&y)[TWW][16], float (&sa)[KC], v4i (&qv)[NT], int8_t* tap, size_t tap_row) {
         float am = 0.0f;
 #pragma unroll
-        for (int i = 0; i < TW; i++)
+        for (int i = 0; i < TWW; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++) am = __builtin_fmaxf(am, __builtin_fabsf(y[i][r]));
-        xch[2 * 256 + wave * 64 + lane] = am;
+        xch[2 * XS + wave * 64 + lane] = am;
         lds_barrier();
 #pragma unroll
         for (int c = 0; c < KC; c++) {
-            float m = 0.0f;
+            float m = 0.0f;   // the maximum is exact in any order: every wave of the chunk's quarters
 #pragma unroll
-            for (int w = c * WPC; w < (c + 1) * WPC; w++) m = __builtin_fmaxf(m, xch[2 * 256 + w * 64 + lane]);
+            for (int w = c * WPC; w < (c + 1) * WPC; w++)
+#pragma unroll
+                for (int u = 0; u < SUB; u++) m = __builtin_fmaxf(m, xch[2 * XS + (w + 4 * u) * 64 + lane]);
             m = __builtin_fmaxf(m, partner(m, g));
             sa[c] = m > 0.0f ? m / (FP8 ? 8.0f : 127.0f) : 1.0f;
         }
-        const float so = KC == 1 ? sa[0] : (wave < WPC ? sa[0] : sa[KC - 1]);
+        const float so = KC == 1 ? sa[0] : (q < WPC ? sa[0] : sa[KC - 1]);
         const float inv = 1.0f / so;
 #pragma unroll
-        for (int i = 0; i < TW; i++) {
+        for (int i = 0; i < TWW; i++) {
             v4i w;
 #pragma unroll
             for (int j = 0; j < 4; j++)
                 w[j] = (int)quant4<FP8>(y[i][4 * j], y[i][4 * j + 1], y[i][4 * j + 2], y[i][4 * j + 3], so, inv);
-            *reinterpret_cast<v4i*>(act + (TW * wave + i) * FRAG + lane * 16) = w;
+            *reinterpret_cast<v4i*>(act + (TW * q + t0 + i) * FRAG + lane * 16) = w;
             if (TAPS && tap)
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    *reinterpret_cast<int*>(tap + (tap_row * T + t) * D + 32 * (TW * wave + i) + 8 * j + 4 * g) = w[j];
+                    *reinterpret_cast<int*>(tap + (tap_row * T + t) * D + 32 * (TW * q + t0 + i) + 8 * j + 4 * g) = w[j];
         }
         lds_barrier();
 #pragma unroll
-        for (int n = 0; n < NT; n++) q[n] = *reinterpret_cast<const v4i*>(act + n * FRAG + lane * 16);
+        for (int n = 0; n < NT; n++) qv[n] = *reinterpret_cast<const v4i*>(act + n * FRAG + lane * 16);
     };
 
     // ---- start the weight stream and the first layer's parameters ------------------------------
     if constexpr (TWIN) {
 #pragma unroll
-        for (int j = 0; j < NSETS - 1; j++) load_half(j, j);
+        for (int j = 0; j < NSETS - 1; j++) fetch_half(j, 0, BPW);
     } else {
 #pragma unroll
         for (int j = 0; j < SLOTS; j++) issue_block(j, j);
@@ -256,16 +314,16 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     }
 
     // ---- embedding (this wave's channels) --------------------------------------------------------
-    float x[TW][16];
+    float x[TWW][16];
     const unsigned word = a.boards[(size_t)b * T + t];
     const int ctrl = a.control[b];
     const unsigned alive = (unsigned)__ballot(((word >> 11) & 1) == 0 && g == 0);
     if (TAPS && a.taps.x_in) {
 #pragma unroll
-        for (int i = 0; i < TW; i++)
+        for (int i = 0; i < TWW; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const v4f v = ldg4(a.taps.x_in + ((size_t)b * T + t) * D + 32 * (TW * wave + i) + 8 * j + 4 * g);
+                const v4f v = ldg4(a.taps.x_in + ((size_t)b * T + t) * D + 32 * (TW * q + t0 + i) + 8 * j + 4 * g);
 #pragma unroll
                 for (int k = 0; k < 4; k++) x[i][4 * j + k] = v[k];
             }
@@ -278,14 +336,14 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
         int ts = ((word >> 6) & 7) * 2 + ((word >> 9) & 1);
         ts = ts > 11 ? 11 : ts;
         const int ct = ((word >> 10) & 1) * 2 + stm;
-        const int own = CW * wave + 4 * g;
+        const int own = CW * q + 32 * t0 + 4 * g;
         const float* e_sq = gp + C::G_SQ + (word & 63) * D + own;
         const float* e_ts = gp + C::G_TS + ts * D + own;
         const float* e_ct = gp + C::G_CT + ct * D + own;
         const float* e_ck = gp + C::G_CLOCK + clock * D + own;
         const float* e_rp = gp + C::G_REP + rp * D + own;
 #pragma unroll
-        for (int i = 0; i < TW; i++)
+        for (int i = 0; i < TWW; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int c = 32 * i + 8 * j;
@@ -302,10 +360,10 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     }
     if (TAPS && a.taps.embed)
 #pragma unroll
-        for (int i = 0; i < TW; i++)
+        for (int i = 0; i < TWW; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++)
-                a.taps.embed[((size_t)b * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = x[i][r];
+                a.taps.embed[((size_t)b * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = x[i][r];
 
     wait_vm<0>();   // the parameters (and the first ring slots) have landed
     if constexpr (!TWIN) read_slot(0);
@@ -314,21 +372,23 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
         const int li = l - a.l0;
         const size_t bl = (size_t)b * nl_run + li;   // tap row
         const int lnext = l + 1 < a.l1 ? l + 1 : l;  // after the last layer the same slice is fetched again
-        // Multiply by block k of this wave's layer.
+        // Multiply by the wave's k-th block of this layer (its own count: see block_at).
         // TWIN: its two halves sit in register sets 2k % NSETS and (2k + 1) % NSETS; a set is refilled
-        // with the half-block NSETS positions on once it has been consumed.
+        // with the wave's half-block NSETS positions on once it has been consumed.  Four waves: that
+        // runs on into the next layer and, after the last one, into the head blocks.  Eight waves:
+        // after the last layer of the run the same layer is fetched again (and never used).
         // !TWIN: the block is in `fr`; the ring slot it came from is refilled SLOTS blocks ahead,
         // then block k+1 is read from its slot.
-        const int hbase = li * 2 * BPW;
+        const int lbase = li * BPW, lfollow = OCTO ? (lnext - a.l0) * BPW : (li + 1) * BPW;
 #define BF_WMM(SWAP, k, actp)                                                                        \
     ([&]() -> acc_t {                                                                                \
         const v4i* act_ = (actp);                                                                    \
         acc_t r_ = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};                                 \
         if constexpr (TWIN) {                                                                        \
-            load_half(hbase + 2 * (k) + NSETS - 1, (2 * (k) + NSETS - 1) % NSETS);                   \
+            fetch_half(2 * (k) + NSETS - 1, lbase, lfollow);                                         \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
                 r_ = frag_mma<SWAP>(frt[(2 * (k)) % NSETS][s_], act_[s_], r_);                       \
-            load_half(hbase + 2 * (k) + NSETS, (2 * (k) + NSETS) % NSETS);                           \
+            fetch_half(2 * (k) + NSETS, lbase, lfollow);                                             \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
                 r_ = frag_mma<SWAP>(frt[(2 * (k) + 1) % NSETS][s_], act_[4 + s_], r_);               \
         } else {                                                                                     \
@@ -346,8 +406,8 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
         v4i xq[NT];
         float sa[KC];
         {
-            float y[TW][16];
-            layernorm(x, pA + C::A_LN1G, pA + C::A_LN1B, y);
+            float y[TWW][16];
+            layernorm(x, pA + C::A_LN1G + 32 * t0, pA + C::A_LN1B + 32 * t0, y);
             quant_exchange(y, sa, xq, TAPS ? a.taps.qa_qkv : nullptr, bl);
         }
         float sa_tok[KC][16];   // activation scale of token ch(r, g), for the V tiles whose rows are tokens
@@ -359,10 +419,10 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
         // ---- attention over this wave's heads ----------------------------------------------------------
         // !TWIN: software-pipelined -- the three weight GEMMs of head i+1 are issued right after the
         // score MFMAs of head i, so the matrix pipe works through them under head i's softmax.
-        float o[TW][16];
+        float o[TWW][16];
         acc_t accq[KC], acck[KC], accv[KC];
 #pragma unroll
-        for (int i = 0; i < TW; i++) {
+        for (int i = 0; i < TWW; i++) {
             if (TWIN || i == 0) {
 #pragma unroll
                 for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * i + c, &xq[8 * c]);
@@ -371,14 +431,15 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
 #pragma unroll
                 for (int c = 0; c < KC; c++) accv[c] = BF_WMM(true, 3 * KC * i + 2 * KC + c, &xq[8 * c]);
             }
-            const int h = TW * wave + i;
+            const int h = TW * q + t0 + i;
             float qf[16], kf[16], vf[16];
             {
-                const float swq = pA[C::A_SW + i], swk = pA[C::A_SW + TW + i], swv = pA[C::A_SW + 2 * TW + i];
-                const float bv = pA[C::A_BV + 32 * i + t];
+                const int ti = t0 + i;   // this head's tile within the quarter
+                const float swq = pA[C::A_SW + ti], swk = pA[C::A_SW + TW + ti], swv = pA[C::A_SW + 2 * TW + ti];
+                const float bv = pA[C::A_BV + 32 * ti + t];
                 v4f bq[4], bk[4];
-                load_tile16(pA + C::A_BQ + 32 * i, g, bq);
-                load_tile16(pA + C::A_BK + 32 * i, g, bk);
+                load_tile16(pA + C::A_BQ + 32 * ti, g, bq);
+                load_tile16(pA + C::A_BK + 32 * ti, g, bk);
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -408,7 +469,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             v16f sc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
             for (int r = 0; r < 16; r++) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[r], qf[r], sc, 0, 0, 0);
-            if (!TWIN && i + 1 < TW) {
+            if (!TWIN && i + 1 < TWW) {
 #pragma unroll
                 for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * (i + 1) + c, &xq[8 * c]);
 #pragma unroll
@@ -445,18 +506,18 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             v4i oq[NT];
             float so[KC];
             quant_exchange(o, so, oq, TAPS ? a.taps.qa_out : nullptr, bl);
-            constexpr int K0 = 3 * KC * TW;
+            constexpr int K0 = 3 * KC * TWW;
             acc_t acc2[2][KC];
 #pragma unroll
             for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, K0 + c, &oq[8 * c]);
 #pragma unroll
-            for (int i = 0; i < TW; i++) {
-                if (i + 1 < TW)
+            for (int i = 0; i < TWW; i++) {
+                if (i + 1 < TWW)
 #pragma unroll
                     for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, K0 + KC * (i + 1) + c, &oq[8 * c]);
                 v4f bo[4];
-                load_tile16(pA + C::A_BOUT + 32 * i, g, bo);
-                const float sw = pA[C::A_SW + 3 * TW + i];
+                load_tile16(pA + C::A_BOUT + 32 * (t0 + i), g, bo);
+                const float sw = pA[C::A_SW + 3 * TW + t0 + i];
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -468,7 +529,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
                     for (int c = 0; c < KC; c++)
 #pragma unroll
                         for (int r = 0; r < 16; r++)
-                            a.taps.acc_out[((bl * KC + c) * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = accbits(acc2[i & 1][c], r);
+                            a.taps.acc_out[((bl * KC + c) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = accbits(acc2[i & 1][c], r);
             }
         }
         // the attention-phase parameters are dead: fetch the next layer's
@@ -477,32 +538,32 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
 
         // ---- feed-forward --------------------------------------------------------------------------------
         {
-            float y[TW][16];
-            layernorm(x, pB + C::B_LN2G, pB + C::B_LN2B, y);
+            float y[TWW][16];
+            layernorm(x, pB + C::B_LN2G + 32 * t0, pB + C::B_LN2B + 32 * t0, y);
             quant_exchange(y, sa, xq, TAPS ? a.taps.qa_ff1 : nullptr, bl);
         }
-        double o64[TW][16];   // int8: float64 sums over the k-chunks
-        float o32[TW][16];    // e4m3: fp32 sums over the k-tiles
-        constexpr int KF = 3 * KC * TW + KC * TW;   // first feed-forward block of the layer
+        double o64[TWW][16];   // int8: float64 sums over the k-chunks
+        float o32[TWW][16];    // e4m3: fp32 sums over the k-tiles
+        constexpr int KF = 3 * KC * TWW + KC * TWW;   // the wave's first feed-forward block of the layer
 #pragma unroll
         for (int st = 0; st < STEPS; st++) {
-            constexpr int SBLK = 4 * KC + 2 * TW;   // blocks of one step
-            const int k1 = KF + st * SBLK;          // first matmul: four hidden tiles of this wave (half a 256-wide chunk)
-            float sh[2];                            // scales of the step's two chunks
+            constexpr int SBLK = HT * KC + 2 * TWW;   // the wave's blocks of one step
+            const int k1 = KF + st * SBLK;            // first matmul: HT hidden tiles of this wave (of the 16 of a step)
+            float sh[2];                              // scales of the step's two chunks
             {
-                float hf[4][16];
+                float hf[HT][16];
                 float am = 0.0f;
                 acc_t acc2[2][KC];
 #pragma unroll
                 for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + c, &xq[8 * c]);
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    if (i + 1 < 4)
+                for (int i = 0; i < HT; i++) {
+                    if (i + 1 < HT)
 #pragma unroll
                         for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, k1 + KC * (i + 1) + c, &xq[8 * c]);
                     v4f b1[4];
-                    load_tile16(pB + C::B_BFF1 + 128 * st + 32 * i, g, b1);
-                    const float sw = pB[C::B_SW + 4 * st + i];
+                    load_tile16(pB + C::B_BFF1 + 128 * st + 32 * (h0 + i), g, b1);
+                    const float sw = pB[C::B_SW + 4 * st + h0 + i];
 #pragma unroll
                     for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -517,50 +578,54 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
                         for (int c = 0; c < KC; c++)
 #pragma unroll
                             for (int r = 0; r < 16; r++)
-                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * wave + 32 * i + ch(r, g)] = accbits(acc2[i & 1][c], r);
+                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + ch(r, g)] = accbits(acc2[i & 1][c], r);
                 }
                 // quantiser over the 256-wide chunk this wave shares with its neighbour (waves 0,1: first
                 // chunk of the step; 2,3: second).  int8: unsigned, bytes stored as q - 128 for the signed
                 // MFMA; e4m3: the ordinary signed quantiser (the values are non-negative)
-                xch[2 * 256 + wave * 64 + lane] = am;
+                xch[2 * XS + wave * 64 + lane] = am;
                 lds_barrier();
 #pragma unroll
                 for (int c = 0; c < 2; c++) {
-                    float m = __builtin_fmaxf(xch[2 * 256 + (2 * c) * 64 + lane], xch[2 * 256 + (2 * c + 1) * 64 + lane]);
+                    float m = 0.0f;   // hidden values are >= 0
+#pragma unroll
+                    for (int u = 0; u < SUB; u++)
+                        m = __builtin_fmaxf(m, __builtin_fmaxf(xch[2 * XS + (2 * c + 4 * u) * 64 + lane],
+                                                               xch[2 * XS + (2 * c + 1 + 4 * u) * 64 + lane]));
                     m = __builtin_fmaxf(m, partner(m, g));
                     sh[c] = m > 0.0f ? m / (FP8 ? 8.0f : 255.0f) : 1.0f;
                 }
-                const float s8 = wave < 2 ? sh[0] : sh[1];
+                const float s8 = q < 2 ? sh[0] : sh[1];
                 const float inv = 1.0f / s8;
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
+                for (int i = 0; i < HT; i++) {
                     v4i w;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const unsigned u = quant4<FP8>(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
                         if (TAPS && a.taps.qa_ff2)
-                            *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 512 * st + 128 * wave + 32 * i + 8 * j + 4 * g) = u;
+                            *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + 8 * j + 4 * g) = u;
                         w[j] = (int)(FP8 ? u : (u ^ 0x80808080u));
                     }
-                    *reinterpret_cast<v4i*>(hid + (4 * wave + i) * FRAG + lane * 16) = w;
+                    *reinterpret_cast<v4i*>(hid + (4 * q + h0 + i) * FRAG + lane * 16) = w;
                 }
             }
             lds_barrier();
             // second matmul, chunk-major: one chunk of the hidden row (eight fragments) serves this
             // wave's TW output tiles; the float64 sums over the chunks stay in chunk order
-            const int k2 = k1 + 4 * KC;
+            const int k2 = k1 + HT * KC;
             acc_t acc2[2];
             v4i hqc[8];
 #pragma unroll
             for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + s * FRAG + lane * 16);
             acc2[0] = BF_WMM(false, k2, &hqc[0]);
 #pragma unroll
-            for (int idx = 0; idx < 2 * TW; idx++) {
-                const int c = idx / TW, i = idx % TW;
+            for (int idx = 0; idx < 2 * TWW; idx++) {
+                const int c = idx / TWW, i = idx % TWW;
                 v4i ws[4];
-                if (!FP8) load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * i, g, ws);
-                if (idx + 1 < 2 * TW) {
-                    if ((idx + 1) % TW == 0)
+                if (!FP8) load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * (t0 + i), g, ws);
+                if (idx + 1 < 2 * TWW) {
+                    if ((idx + 1) % TWW == 0)
 #pragma unroll
                         for (int s = 0; s < 8; s++)
                             hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * (c + 1) + s) * FRAG + lane * 16);
@@ -569,13 +634,13 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
                 const acc_t acc = acc2[idx & 1];
                 if constexpr (FP8) {
                     // descale each 256-deep tile with its own scales, fp32 sum over the tiles
-                    const float sw = pB[C::B_SW + 16 + i * KCF + 2 * st + c];
+                    const float sw = pB[C::B_SW + 16 + (t0 + i) * KCF + 2 * st + c];
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const float part = (accf(acc, r) * sh[c]) * sw;
                         o32[i][r] = (st == 0 && c == 0) ? part : o32[i][r] + part;
                         if (TAPS && a.taps.acc_ff2)
-                            a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = accbits(acc, r);
+                            a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = accbits(acc, r);
                     }
                     pin16(o32[i]);
                 } else {
@@ -588,7 +653,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
                             o64[i][4 * j + k] = (st == 0 && c == 0) ? (double)full * sc
                                                                     : __builtin_fma((double)full, sc, o64[i][4 * j + k]);
                             if (TAPS && a.taps.acc_ff2)
-                                a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * wave + i) + 8 * j + 4 * g + k] = full;
+                                a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * q + t0 + i) + 8 * j + 4 * g + k] = full;
                         }
 #pragma unroll
                     for (int r = 0; r < 16; r++) pin(o64[i][r]);
@@ -596,10 +661,10 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             }
         }
 #pragma unroll
-        for (int i = 0; i < TW; i++) {
+        for (int i = 0; i < TWW; i++) {
             v4f b2[4];
-            load_tile16(pB + C::B_BFF2 + 32 * i, g, b2);
-            const float sw = pB[C::B_SW + 16 + i];
+            load_tile16(pB + C::B_BFF2 + 32 * (t0 + i), g, b2);
+            const float sw = pB[C::B_SW + 16 + t0 + i];
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -615,10 +680,10 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
 #undef BF_WMM
         if (TAPS && a.taps.resid)
 #pragma unroll
-            for (int i = 0; i < TW; i++)
+            for (int i = 0; i < TWW; i++)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    a.taps.resid[(bl * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = x[i][r];
+                    a.taps.resid[(bl * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = x[i][r];
     }
 
     // ---- final norm and heads --------------------------------------------------------------------------
@@ -626,7 +691,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     // the blocks of the next layer there: then restart the stream at the head blocks.
     const int hseq0 = (a.n_layers - a.l0) * BPW;
     wait_vm<0>();   // also: no parameter copy is still landing where the normalised stream goes
-    if (a.l1 != a.n_layers) {
+    if (OCTO || a.l1 != a.n_layers) {
         if constexpr (TWIN) {
 #pragma unroll
             for (int j = 0; j < NSETS - 1; j++) load_half(2 * hseq0 + j, j);
@@ -638,28 +703,32 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             read_slot(0);
         }
     }
-    float hn[TW][16];
-    layernorm(x, gp + C::G_NFG + CW * wave, gp + C::G_NFB + CW * wave, hn);
+    float hn[TWW][16];
+    layernorm(x, gp + C::G_NFG + CW * q + 32 * t0, gp + C::G_NFB + CW * q + 32 * t0, hn);
     if (TAPS && a.taps.normed)
 #pragma unroll
-        for (int i = 0; i < TW; i++)
+        for (int i = 0; i < TWW; i++)
 #pragma unroll
             for (int r = 0; r < 16; r++)
-                a.taps.normed[((size_t)b * T + t) * D + 32 * (TW * wave + i) + ch(r, g)] = hn[i][r];
+                a.taps.normed[((size_t)b * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = hn[i][r];
     // publish as B-operand fragments (n, j): lane holds the four floats of register quad j
     float* const hnb = reinterpret_cast<float*>(hid);
 #pragma unroll
-    for (int i = 0; i < TW; i++)
+    for (int i = 0; i < TWW; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const v4f v = {hn[i][4 * j], hn[i][4 * j + 1], hn[i][4 * j + 2], hn[i][4 * j + 3]};
-            *reinterpret_cast<v4f*>(hnb + (((TW * wave + i) * 4 + j) * 64 + lane) * 4) = v;
+            *reinterpret_cast<v4f*>(hnb + (((TW * q + t0 + i) * 4 + j) * 64 + lane) * 4) = v;
         }
     lds_barrier();
-    // wave m multiplies head tile m (rows 32m..32m+31 of [policy; promo; value; 0]) over the whole
-    // width, one fused-multiply-add chain in (tile, quad, element) order; wave 3's tile is zero
+    // The first wave of quarter m multiplies head tile m (rows 32m..32m+31 of [policy; promo;
+    // value; 0]) over the whole width, one fused-multiply-add chain in (tile, quad, element) order;
+    // quarter 3's tile is zero.  With eight waves the second wave of a quarter has nothing to
+    // do here but meet the barrier of the argmax exchange.
+    const bool heads_here = !OCTO || sub == 0;
     v16f head = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    if constexpr (TWIN) {
+    if (!heads_here) {
+    } else if constexpr (TWIN) {
 #pragma unroll
         for (int hi = 0; hi < 2 * HB; hi++) {          // half-block = the four fragments (n = hi, q = 0..3)
             // the stream is padded by one block: two half-blocks past the last head block exist
@@ -692,7 +761,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     }
 
     // value: king token of the side to move, lane half 1 of head tile 2 holds rows 68..70
-    if (wave == 2) {
+    if (heads_here && q == 2) {
         const int king = ctrl < 0 ? 31 : 15;
         if (lane == 32 + king) {
             float v;
@@ -719,7 +788,7 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     // policy (waves 0 and 1: squares 0..31 and 32..63), optional legal-move AND and argmax
     float bv = -__builtin_inff();
     int bi = 0x7fffffff;
-    if (wave < 2) {
+    if (heads_here && q < 2) {
         unsigned long long mw = ~0ull;
         if (a.mask) mw = a.mask[(size_t)b * T + t];
 #pragma unroll
@@ -727,13 +796,13 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             float v[4];
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const int sq = 32 * wave + 8 * j + 4 * g + k;
+                const int sq = 32 * q + 8 * j + 4 * g + k;
                 const bool legal = (mw >> sq) & 1ull;
                 v[k] = legal ? head[4 * j + k] : -__builtin_inff();
                 // squares are visited in increasing order within a lane, so '>' keeps the lowest
                 if (legal && (bi == 0x7fffffff || v[k] > bv)) { bv = v[k]; bi = t * 64 + sq; }
             }
-            const size_t at = ((size_t)b * T + t) * 64 + 32 * wave + 8 * j + 4 * g;
+            const size_t at = ((size_t)b * T + t) * 64 + 32 * q + 8 * j + 4 * g;
             if (a.out_fp32) {
                 const v4f vv = {v[0], v[1], v[2], v[3]};
                 *reinterpret_cast<v4f*>((float*)a.policy + at) = vv;
@@ -753,9 +822,9 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
             bi = take ? oi : bi;
         }
         // the two policy waves' winners meet in the exchange area (its last use was long ago)
-        if (lane == 0) {
-            xch[wave * 2] = bv;
-            xch[wave * 2 + 1] = __int_as_float(bi);
+        if (heads_here && lane == 0) {
+            xch[q * 2] = bv;
+            xch[q * 2 + 1] = __int_as_float(bi);
         }
         lds_barrier();
         if (wave == 0 && lane == 0) {
@@ -768,18 +837,18 @@ __global__ __launch_bounds__(THREADS, TWIN ? BF_TWIN_OCC : 1) void board_kernel(
     }
 }
 
-template <int DM, bool TAPS, bool TWIN, bool FP8 = false>
+template <int DM, bool TAPS, bool TWIN, bool FP8 = false, bool OCTO = false>
 hipError_t launch_board(const KArgs& k, hipStream_t stream) {
     // more than 64 KiB of dynamic LDS has to be requested once per kernel (per thread: cheap)
     static thread_local bool lds_set = false;
-    constexpr int lds_bytes = Cfg<DM, TWIN>::LDS_BYTES;
+    constexpr int lds_bytes = Cfg<DM, TWIN, OCTO>::LDS_BYTES;
     if (!lds_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&board_kernel<DM, TAPS, TWIN, FP8>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&board_kernel<DM, TAPS, TWIN, FP8, OCTO>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess) return e;
         lds_set = true;
     }
-    hipLaunchKernelGGL((board_kernel<DM, TAPS, TWIN, FP8>), dim3(k.n), dim3(THREADS), lds_bytes, stream, k);
+    hipLaunchKernelGGL((board_kernel<DM, TAPS, TWIN, FP8, OCTO>), dim3(k.n), dim3(OCTO ? 2 * THREADS : THREADS), lds_bytes, stream, k);
     return hipGetLastError();
 }
 

@@ -29,9 +29,9 @@ static bool shape512(const bf_shape* s) {
 
 static bool board_shape_ok(const bf_shape* s) { return shape_ok(s) || shape512(s); }
 
-// AUTO runs one workgroup per compute unit (lowest latency per position) up to this many
-// positions, which is one per compute unit of an MI355X; above it, two workgroups per compute
-// unit (highest throughput).
+// AUTO runs one workgroup per compute unit (lowest latency per position; eight wavefronts per
+// position where that form exists, else four) up to this many positions, which is one per
+// compute unit of an MI355X; above it, two workgroups per compute unit (highest throughput).
 static const int64_t kBoardMaxN = 256;
 
 template <int DM>
@@ -103,6 +103,7 @@ static int choose_kernel(const bf_eval_args* a) {
     // the board blobs are packed for one format; the 512-wide network runs int8 only
     const bool board_can = have_board && (a->quant == BF_QUANT_INT8 || shape_ok(&a->shape));
     const bool twin_can = have_board && shape_ok(&a->shape);
+    const bool octo_can = twin_can && a->quant == BF_QUANT_INT8;
     switch (a->kernel) {
     case BF_KERNEL_QUAD:
         if (!quad_can) return fail(BF_ERR_UNSUPPORTED, "the four-positions-per-workgroup kernel needs the 256-wide network and wstream/fparams");
@@ -114,14 +115,21 @@ static int choose_kernel(const bf_eval_args* a) {
         if (!twin_can)
             return fail(BF_ERR_UNSUPPORTED, "the two-workgroups-per-compute-unit kernel needs the 256-wide network and board_wstream/board_fparams");
         return BF_KERNEL_TWIN;
+    case BF_KERNEL_OCTO:
+        if (!octo_can)
+            return fail(BF_ERR_UNSUPPORTED, "the eight-wavefronts-per-position kernel needs the 256-wide network, board_wstream/board_fparams and the int8 format");
+        return BF_KERNEL_OCTO;
     case BF_KERNEL_AUTO:
-        if (board_can) return (twin_can && a->n > kBoardMaxN) ? BF_KERNEL_TWIN : BF_KERNEL_BOARD;
+        if (board_can) {
+            if (twin_can && a->n > kBoardMaxN) return BF_KERNEL_TWIN;
+            return octo_can ? BF_KERNEL_OCTO : BF_KERNEL_BOARD;
+        }
         if (quad_can) return BF_KERNEL_QUAD;
         return fail(BF_ERR_ARGUMENT, shape512(&a->shape)
                         ? "the 512-wide network runs on the one-position-per-workgroup kernel: int8, board_wstream/board_fparams required"
                         : "wstream/fparams must not be NULL");
     default:
-        return fail(BF_ERR_ARGUMENT, "kernel must be BF_KERNEL_AUTO, BF_KERNEL_QUAD, BF_KERNEL_BOARD or BF_KERNEL_TWIN");
+        return fail(BF_ERR_ARGUMENT, "kernel must be BF_KERNEL_AUTO, BF_KERNEL_QUAD, BF_KERNEL_BOARD, BF_KERNEL_TWIN or BF_KERNEL_OCTO");
     }
 }
 
@@ -130,7 +138,7 @@ extern "C" int bf_kernel_choice(const bf_eval_args* args) { return choose_kernel
 static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     *kind = choose_kernel(a);
     if (*kind < 0) return *kind;
-    const bool board = *kind == BF_KERNEL_BOARD || *kind == BF_KERNEL_TWIN;
+    const bool board = *kind == BF_KERNEL_BOARD || *kind == BF_KERNEL_TWIN || *kind == BF_KERNEL_OCTO;
     if (a->n < 1 || a->n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
     if (!a->boards || !a->control || !a->rep) return fail(BF_ERR_ARGUMENT, "boards/control/rep must not be NULL");
     if (!a->policy || !a->promo || !a->value) return fail(BF_ERR_ARGUMENT, "policy/promo/value must not be NULL");
@@ -170,7 +178,10 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
 static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream_t stream) {
     const int grid = (k.n + bf::WAVES - 1) / bf::WAVES;
     hipError_t e;
-    if (kind == BF_KERNEL_TWIN) {
+    if (kind == BF_KERNEL_OCTO) {
+        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
+        e = a->taps ? bf::launch_octo256_taps(k, stream) : bf::launch_octo256(k, stream);
+    } else if (kind == BF_KERNEL_TWIN) {
         if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
         if (a->quant == BF_QUANT_E4M3)
             e = a->taps ? bf::launch_twin256_fp8_taps(k, stream) : bf::launch_twin256_fp8(k, stream);

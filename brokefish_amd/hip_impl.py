@@ -449,7 +449,7 @@ class FusedEncoder:
 
     D, DFF, T, H = 256, 1024, 32, 8
     SHAPES = ((256, 1024, 8), (512, 2048, 16))     # (d_model, d_ff, heads) the library carries
-    KERNELS = {"auto": 0, "quad": 1, "board": 2, "twin": 3}   # enum bf_kernel
+    KERNELS = {"auto": 0, "quad": 1, "board": 2, "twin": 3, "octo": 4}   # enum bf_kernel
     ACC_DTYPES = ("fp16", "fp32")
     n_value = 1
     vmode = 0
@@ -498,7 +498,9 @@ class FusedEncoder:
         wide = self.d_model != self.D
         if wide and fp8:
             raise NotImplementedError("the 512-wide network runs in int8 only")
-        if wide and kernel in ("quad", "twin"):
+        if fp8 and kernel == "octo":
+            raise NotImplementedError("the eight-wavefront kernel runs in int8 only")
+        if wide and kernel in ("quad", "twin", "octo"):
             raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernel "
                                       "(kernel='board' or 'auto') only")
         if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
@@ -534,7 +536,7 @@ class FusedEncoder:
         # kernel (int8; small launches of the 256-wide network and the 512-wide network).
         self.kernel = kernel
         self.wstream = self.fparams = self.board_wstream = self.board_fparams = None
-        if not wide and kernel not in ("board", "twin"):
+        if not wide and kernel not in ("board", "twin", "octo"):
             wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value,
                                             fmt="e4m3" if self.fp8 else "int8")
             if wstream.size != self._lib.bf_wstream_bytes(C.byref(self._shape)) or \
@@ -557,7 +559,7 @@ class FusedEncoder:
     def label(self) -> str:
         fmt = "e4m3" if self.fp8 else "int8"
         names = {"quad": "4 boards/workgroup", "board": "1 board/workgroup",
-                 "twin": "1 board/workgroup, 2 workgroups/CU"}
+                 "twin": "1 board/workgroup, 2 workgroups/CU", "octo": "1 board/workgroup of 8 wavefronts"}
         if self.kernel != "auto":
             per = names[self.kernel]
         elif self.board_wstream is None:
@@ -636,7 +638,7 @@ class FusedEncoder:
         rc = self._lib.bf_kernel_choice(C.byref(a))
         if rc < 0:
             raise RuntimeError(f"bf_kernel_choice failed ({rc}): {self._lib.bf_last_error().decode()}")
-        return {1: "quad", 2: "board", 3: "twin"}[rc]
+        return {1: "quad", 2: "board", 3: "twin", 4: "octo"}[rc]
 
     def forward_expand(self, boards, control, rep, mask=None, max_edges: int = 96, active=None, out=None):
         """``forward_full`` followed on the same stream by the search's expand step

@@ -40,24 +40,28 @@ enum bf_quant {
     BF_QUANT_E4M3 = 1
 };
 
-/* Three kernels compute the same function.
+/* Four kernels compute the same function.
  *   QUAD   four positions per workgroup, one wavefront each, weights shared through LDS; carries
  *          the phase profile (256-wide network, int8 and e4m3).
  *   BOARD  one position per workgroup, the four wavefronts split the model width; one workgroup
- *          per compute unit: the lowest latency per position (launches that cannot fill the GPU)
- *          and the only kernel the 512-wide network fits.
+ *          per compute unit: low latency per position (launches that cannot fill the GPU) and
+ *          the only kernel the 512-wide network fits.
  *   TWIN   the BOARD decomposition shaped so that two workgroups share a compute unit (each SIMD
  *          holds two wavefronts that cover each other's waits): the highest throughput
  *          (256-wide network).
- * BOARD and TWIN read the same blobs (board_wstream / board_fparams).  The 256-wide network runs
- * in int8 and e4m3 on all three, the 512-wide network in int8 on BOARD.  For the 256-wide network
- * the three kernels return bit-identical results in either format, so AUTO may pick by batch
- * size. */
+ *   OCTO   the BOARD decomposition with eight wavefronts per position (two per quarter of the
+ *          width, each taking half of the quarter's tiles), one workgroup per compute unit: the
+ *          lowest latency per position (256-wide network, int8).
+ * BOARD, TWIN and OCTO read the same blobs (board_wstream / board_fparams).  The 256-wide network
+ * runs in int8 on all four and in e4m3 on QUAD, BOARD and TWIN; the 512-wide network in int8 on
+ * BOARD.  For the 256-wide network the kernels return bit-identical results in either format, so
+ * AUTO may pick by batch size. */
 enum bf_kernel {
     BF_KERNEL_AUTO = 0,
     BF_KERNEL_QUAD = 1,
     BF_KERNEL_BOARD = 2,
-    BF_KERNEL_TWIN = 3
+    BF_KERNEL_TWIN = 3,
+    BF_KERNEL_OCTO = 4
 };
 
 /* Sizes of one 32-token position, fixed by the position format
@@ -152,9 +156,9 @@ typedef struct {
      * paying for the leaves that need no evaluation (BOARD / TWIN: the workgroup exits at once;
      * QUAD: the wavefront runs on, storing nothing) */
     const uint8_t* active;
-    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: BOARD for the 512-wide
-                             * network and for n <= bf_board_max_n(), TWIN above; without
-                             * them QUAD */
+    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: for n <= bf_board_max_n()
+                             * OCTO (int8, 256-wide network) or BOARD (e4m3; the 512-wide
+                             * network at any n), TWIN above; without them QUAD */
 } bf_eval_args;
 
 /* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */

@@ -86,19 +86,19 @@ def test_kernel_choice_follows_shape_blobs_and_batch_size():
     a.wstream = a.fparams = a.board_wstream = a.board_fparams = 16      # only tested for NULL here
     cut = lib.bf_board_max_n()
     assert cut == 256                                                    # one position per compute unit
-    for n, want in ((1, 2), (cut, 2), (cut + 1, 3), (4096, 3)):          # BOARD up to the cut, TWIN above
+    for n, want in ((1, 4), (cut, 4), (cut + 1, 3), (4096, 3)):          # OCTO up to the cut, TWIN above
         a.n = n
         assert lib.bf_kernel_choice(ctypes.byref(a)) == want
-    for forced in (1, 2, 3):
+    for forced in (1, 2, 3, 4):
         a.n, a.kernel = 4096, forced
         assert lib.bf_kernel_choice(ctypes.byref(a)) == forced
-    a.kernel, a.quant = 0, 1                                            # e4m3: the same rule
+    a.kernel, a.quant = 0, 1                                            # e4m3: BOARD up to the cut
     for n, want in ((1, 2), (cut, 2), (cut + 1, 3), (4096, 3)):
         a.n = n
         assert lib.bf_kernel_choice(ctypes.byref(a)) == want
-    for forced in (1, 2, 3):
+    for forced, want in ((1, 1), (2, 2), (3, 3), (4, -2)):
         a.kernel = forced
-        assert lib.bf_kernel_choice(ctypes.byref(a)) == forced
+        assert lib.bf_kernel_choice(ctypes.byref(a)) == want
     a.kernel, a.quant, a.board_wstream = 0, 0, None                     # no board blobs: always quad
     a.n = 1
     assert lib.bf_kernel_choice(ctypes.byref(a)) == 1
@@ -106,7 +106,7 @@ def test_kernel_choice_follows_shape_blobs_and_batch_size():
     a.board_wstream = 16
     a.n = 100000
     assert lib.bf_kernel_choice(ctypes.byref(a)) == 2
-    for forced in (1, 3):
+    for forced in (1, 3, 4):
         a.kernel = forced
         assert lib.bf_kernel_choice(ctypes.byref(a)) == -2
     a.kernel, a.quant = 2, 1                                            # ... and in int8 only

@@ -33,7 +33,7 @@ def _make(d, heads, layers, nv=1, seed=0):
 @pytest.fixture(scope="module")
 def base():
     net, sd = _make(256, 8, 8)
-    return (net, sd, {k: encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=k) for k in ("board", "twin")},
+    return (net, sd, {k: encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=k) for k in ("board", "twin", "octo")},
             encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="quad"), c_oracle.COracle(sd))
 
 
@@ -55,7 +55,7 @@ def _bits_equal(a: torch.Tensor, b: np.ndarray) -> bool:
                                         == b.view(np.int32 if b.dtype == np.float32 else b.dtype)).all())
 
 
-@pytest.mark.parametrize("kernel", ["board", "twin"])
+@pytest.mark.parametrize("kernel", ["board", "twin", "octo"])
 def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base, kernel):
     net, sd, boards, quad, co = base
     board = boards[kernel]
@@ -66,7 +66,7 @@ def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base, kerne
         assert _bits_equal(got[k], want[k]), k
 
 
-@pytest.mark.parametrize("kernel", ["board", "twin"])
+@pytest.mark.parametrize("kernel", ["board", "twin", "octo"])
 @pytest.mark.parametrize("nv", [1, 3])
 def test_the_kernels_return_the_same_bits(base, nv, kernel):
     if nv == 1:
@@ -101,7 +101,7 @@ def test_automatic_choice_switches_kernel_by_batch_size_without_changing_results
     net, sd, boards, quad, co = base
     auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
     cut = int(auto._lib.bf_board_max_n())
-    assert auto.kernel_choice(1) == "board" and auto.kernel_choice(cut) == "board"
+    assert auto.kernel_choice(1) == "octo" and auto.kernel_choice(cut) == "octo"
     assert auto.kernel_choice(cut + 1) == "twin" and auto.kernel_choice(4096) == "twin"
     assert "by batch size" in auto.label
     b, c, r, m = positions.random_positions(cut + 4, plies=120, seed=22)
@@ -150,7 +150,7 @@ def test_e4m3_on_the_throughput_kernel_equals_the_four_per_workgroup_kernel(base
         assert torch.equal(x, y[:200])
 
 
-@pytest.mark.parametrize("kernel", ["board", "twin", "quad"])
+@pytest.mark.parametrize("kernel", ["board", "twin", "octo", "quad"])
 def test_skipped_positions_keep_their_output_rows(base, kernel):
     # the search's flat leaf staging: only flagged leaves are evaluated (reference
     # brokefish/search/cuda_impl.py:137-145), the others cost nothing and change nothing
