@@ -1,32 +1,37 @@
-// The evaluator with ONE position per workgroup: the four wavefronts split the model width.
+// The evaluator with ONE position per workgroup: four (or eight) wavefronts split the model width.
 //
-// Wavefront w owns a quarter of the channels of the residual stream (tiles TW*w .. TW*w+TW-1,
-// which are also its attention heads), a quarter of every matmul's output tiles, and streams
+// Quarter q of the width (tiles TW*q .. TW*q+TW-1 of the residual stream, which are also attention
+// heads, and a quarter of every matmul's output tiles) belongs to wavefront q, which streams
 // exactly the weight blocks of those tiles -- privately, so weights need no cross-wave
 // synchronisation.  Quantised activations are exchanged through LDS as ready-made MFMA
 // B-operand fragments; row statistics (LayerNorm sums, quantiser maxima) are exchanged as
-// per-lane partials and combined in wave order, which is the group order of the arithmetic
+// per-lane partials and combined in quarter order, which is the group order of the arithmetic
 // contract in bf_args.h -- so for the 256-wide network this kernel returns bit for bit what the
 // one-wavefront-per-position kernel returns.  The feed-forward block runs in steps of 512 hidden
-// channels: each wave computes four hidden tiles per step, so a 256-wide quantiser chunk spans a
-// pair of waves and its maximum is exchanged; the float64 sums over the chunks stay in order.
+// channels: each quarter computes four hidden tiles per step, so a 256-wide quantiser chunk spans
+// a pair of quarters and its maximum is exchanged; the float64 sums over the chunks stay in order.
 //
-// Two forms, selected by TWIN, with identical results:
+// Three forms, selected by TWIN and OCTO, with identical results:
 //   TWIN = false  one workgroup per compute unit, 512 registers per wave.  Weight blocks stream
 //                 through a private LDS ring per wave (direct-to-LDS loads, SLOTS blocks deep),
-//                 attention is software-pipelined across heads.  Lowest latency per position
-//                 (launches of up to one position per compute unit) and the only form the
-//                 512-wide network fits.
+//                 attention is software-pipelined across heads.  The only form the 512-wide
+//                 network fits.
 //   TWIN = true   two workgroups per compute unit: at most 80 KiB of LDS and 256 registers per
 //                 wave, so every SIMD holds two wavefronts of different positions and one's
 //                 waits (LDS round trips, barriers, MFMA results) are covered by the other's
 //                 work.  Weight fragments go from L2 straight to registers (half a block = four
 //                 fragments at a time, prefetched through a rotation of register sets).
 //                 Highest throughput.
+//   OCTO          (with TWIN's register weight path) eight wavefronts per position, one workgroup
+//                 per compute unit: a quarter belongs to two wavefronts, `sub` = 0 and 1, each
+//                 owning half of the quarter's tiles in every matmul and reading its blocks out
+//                 of the quarter's stream where they lie (block_at).  A quarter's LayerNorm chain
+//                 is started by its first wavefront and continued by its second.  Lowest latency
+//                 per position (launches of up to one position per compute unit).
 //
-// LDS map (bytes): [ring: 4 waves x SLOTS x 8 KiB, absent in the TWIN form] [xch: 3 KiB]
-// [hid: 16 KiB] [act: NT KiB] [par: 4 waves x PW floats].  During the heads the normalised stream
-// (NT*4 KiB, fp32) overlays hid/act/par.
+// LDS map (bytes): [ring: 4 waves x SLOTS x 8 KiB, absent in the TWIN form] [xch: 3 slots of
+// 64 floats per wave] [hid: 16 KiB] [act: NT KiB] [par: PW floats per wave].  During the heads the
+// normalised stream (NT*4 KiB, fp32) overlays hid/act/par.
 #pragma once
 
 #include "bf_device.hip.h"
