@@ -51,6 +51,11 @@
 #ifndef BF_OCTO_SETS
 #define BF_OCTO_SETS 6
 #endif
+// ... on the 512-wide network the form runs whole batches and registers are scarce: four sets
+// (measured at 4096 positions: 12.5 ms; three sets 12.8, six 16.0)
+#ifndef BF_OCTO_SETS_WIDE
+#define BF_OCTO_SETS_WIDE 4
+#endif
 
 namespace bf {
 namespace board {
@@ -155,9 +160,16 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     constexpr int TWW = TW / SUB;             // tiles of the width a wave owns
     constexpr int HT = 4 / SUB;               // hidden tiles a wave computes per feed-forward step
     constexpr int NB = BPW / SUB;             // weight blocks a wave consumes per layer
-    constexpr int NSETS = OCTO ? BF_OCTO_SETS : BF_TWIN_SETS;   // register sets of the prefetch: NSETS - 1 half-blocks in flight
+    // register sets of the prefetch: NSETS - 1 half-blocks in flight
+    constexpr int NSETS = !OCTO ? BF_TWIN_SETS : DM == 256 ? BF_OCTO_SETS : BF_OCTO_SETS_WIDE;
     static_assert(TW % SUB == 0 && (2 * NB) % NSETS == 0, "tiles and register sets must split evenly");
     constexpr int XS = NW * 64;               // floats of one exchange slot
+    // Eight wavefronts on the 512-wide network: a wave has 256 registers and the quantised row alone
+    // would take 64 of them, so the activation fragments are read from LDS at each MFMA instead.
+    constexpr bool ACTL = OCTO && DM == 512;
+    // ... and the next tile's product is issued after a tile's epilogue, not before it (one set of
+    // accumulators instead of two; the SIMD's other wave fills the gap)
+    constexpr bool AHEAD = !ACTL;
     constexpr int HALF = BLOCK / 2;   // four fragments: the unit of the register prefetch (TWIN)
     constexpr int VM_AHEAD = TAPS ? 0 : (SLOTS - 1) * 8;   // ring loads that may stay in flight at a ring wait
     const int lane = threadIdx.x & 63;
@@ -301,8 +313,18 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                     *reinterpret_cast<int*>(tap + (tap_row * T + t) * D + 32 * (TW * q + t0 + i) + 8 * j + 4 * g) = w[j];
         }
         lds_barrier();
+        if constexpr (!ACTL)
 #pragma unroll
-        for (int n = 0; n < NT; n++) qv[n] = *reinterpret_cast<const v4i*>(act + n * FRAG + lane * 16);
+            for (int n = 0; n < NT; n++) qv[n] = *reinterpret_cast<const v4i*>(act + n * FRAG + lane * 16);
+    };
+    // where a block product takes its eight activation fragments from: registers, or (ACTL) LDS
+    struct FragSrc { const v4i* reg; const uint8_t* mem; };
+    auto fragments = [&](const v4i* regs, const uint8_t* buf, int first) -> FragSrc {
+        return FragSrc{regs + first, buf + first * FRAG + lane * 16};
+    };
+    auto fragment = [&](const FragSrc& f, int s) -> v4i {
+        if constexpr (ACTL) return *reinterpret_cast<const v4i*>(f.mem + s * FRAG);
+        else return f.reg[s];
     };
 
     // ---- start the weight stream and the first layer's parameters ------------------------------
@@ -387,20 +409,20 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         const int lbase = li * BPW, lfollow = OCTO ? (lnext - a.l0) * BPW : (li + 1) * BPW;
 #define BF_WMM(SWAP, k, actp)                                                                        \
     ([&]() -> acc_t {                                                                                \
-        const v4i* act_ = (actp);                                                                    \
+        const FragSrc act_ = (actp);                                                                 \
         acc_t r_ = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};                                 \
         if constexpr (TWIN) {                                                                        \
             fetch_half(2 * (k) + NSETS - 1, lbase, lfollow);                                         \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
-                r_ = frag_mma<SWAP>(frt[(2 * (k)) % NSETS][s_], act_[s_], r_);                       \
+                r_ = frag_mma<SWAP>(frt[(2 * (k)) % NSETS][s_], fragment(act_, s_), r_);             \
             fetch_half(2 * (k) + NSETS, lbase, lfollow);                                             \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
-                r_ = frag_mma<SWAP>(frt[(2 * (k) + 1) % NSETS][s_], act_[4 + s_], r_);               \
+                r_ = frag_mma<SWAP>(frt[(2 * (k) + 1) % NSETS][s_], fragment(act_, 4 + s_), r_);     \
         } else {                                                                                     \
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                       \
             issue_block(li * BPW + (k) + SLOTS, (k) % SLOTS);                                        \
             _Pragma("unroll") for (int s_ = 0; s_ < 8; s_++)                                         \
-                r_ = frag_mma<SWAP>(fr[s_], act_[s_], r_);                                           \
+                r_ = frag_mma<SWAP>(fr[s_], fragment(act_, s_), r_);                                 \
             wait_vm<VM_AHEAD>();                                                                     \
             read_slot(((k) + 1) % SLOTS);                                                            \
         }                                                                                            \
@@ -416,10 +438,11 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             quant_exchange(y, sa, xq, TAPS ? a.taps.qa_qkv : nullptr, bl);
         }
         float sa_tok[KC][16];   // activation scale of token ch(r, g), for the V tiles whose rows are tokens
+        if constexpr (AHEAD)
 #pragma unroll
-        for (int c = 0; c < KC; c++)
+            for (int c = 0; c < KC; c++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) sa_tok[c][r] = __shfl(sa[c], ch(r, g));
+                for (int r = 0; r < 16; r++) sa_tok[c][r] = __shfl(sa[c], ch(r, g));
 
         // ---- attention over this wave's heads ----------------------------------------------------------
         // !TWIN: software-pipelined -- the three weight GEMMs of head i+1 are issued right after the
@@ -428,13 +451,13 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         acc_t accq[KC], acck[KC], accv[KC];
 #pragma unroll
         for (int i = 0; i < TWW; i++) {
-            if (TWIN || i == 0) {
+            if (AHEAD && (TWIN || i == 0)) {
 #pragma unroll
-                for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * i + c, &xq[8 * c]);
+                for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * i + c, fragments(xq, act, 8 * c));
 #pragma unroll
-                for (int c = 0; c < KC; c++) acck[c] = BF_WMM(false, 3 * KC * i + KC + c, &xq[8 * c]);
+                for (int c = 0; c < KC; c++) acck[c] = BF_WMM(false, 3 * KC * i + KC + c, fragments(xq, act, 8 * c));
 #pragma unroll
-                for (int c = 0; c < KC; c++) accv[c] = BF_WMM(true, 3 * KC * i + 2 * KC + c, &xq[8 * c]);
+                for (int c = 0; c < KC; c++) accv[c] = BF_WMM(true, 3 * KC * i + 2 * KC + c, fragments(xq, act, 8 * c));
             }
             const int h = TW * q + t0 + i;
             float qf[16], kf[16], vf[16];
@@ -445,18 +468,33 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 v4f bq[4], bk[4];
                 load_tile16(pA + C::A_BQ + 32 * ti, g, bq);
                 load_tile16(pA + C::A_BK + 32 * ti, g, bk);
+                // !AHEAD: one product at a time, descaled before the next one starts
+                if constexpr (!AHEAD)
+#pragma unroll
+                    for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * i + c, fragments(xq, act, 8 * c));
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        qf[4 * j + k] = chunk_sum<KC>(accq, 4 * j + k, sa) * swq + bq[j][k];
-                        kf[4 * j + k] = chunk_sum<KC>(acck, 4 * j + k, sa) * swk + bk[j][k];
-                    }
+                    for (int k = 0; k < 4; k++) qf[4 * j + k] = chunk_sum<KC>(accq, 4 * j + k, sa) * swq + bq[j][k];
+                if constexpr (!AHEAD) {
+                    pin16(qf);
+#pragma unroll
+                    for (int c = 0; c < KC; c++) acck[c] = BF_WMM(false, 3 * KC * i + KC + c, fragments(xq, act, 8 * c));
+                }
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int k = 0; k < 4; k++) kf[4 * j + k] = chunk_sum<KC>(acck, 4 * j + k, sa) * swk + bk[j][k];
+                if constexpr (!AHEAD) {
+                    pin16(kf);
+#pragma unroll
+                    for (int c = 0; c < KC; c++) accv[c] = BF_WMM(true, 3 * KC * i + 2 * KC + c, fragments(xq, act, 8 * c));
+                }
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     float st[KC];
 #pragma unroll
-                    for (int c = 0; c < KC; c++) st[c] = sa_tok[c][r];
+                    for (int c = 0; c < KC; c++) st[c] = AHEAD ? sa_tok[c][r] : __shfl(sa[c], ch(r, g));
                     vf[r] = chunk_sum<KC>(accv, r, st) * swv + bv;
                 }
                 if (TAPS && a.taps.acc_qkv)
@@ -476,11 +514,11 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             for (int r = 0; r < 16; r++) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[r], qf[r], sc, 0, 0, 0);
             if (!TWIN && i + 1 < TWW) {
 #pragma unroll
-                for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * (i + 1) + c, &xq[8 * c]);
+                for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * (i + 1) + c, fragments(xq, act, 8 * c));
 #pragma unroll
-                for (int c = 0; c < KC; c++) acck[c] = BF_WMM(false, 3 * KC * (i + 1) + KC + c, &xq[8 * c]);
+                for (int c = 0; c < KC; c++) acck[c] = BF_WMM(false, 3 * KC * (i + 1) + KC + c, fragments(xq, act, 8 * c));
 #pragma unroll
-                for (int c = 0; c < KC; c++) accv[c] = BF_WMM(true, 3 * KC * (i + 1) + 2 * KC + c, &xq[8 * c]);
+                for (int c = 0; c < KC; c++) accv[c] = BF_WMM(true, 3 * KC * (i + 1) + 2 * KC + c, fragments(xq, act, 8 * c));
             }
             float p[16];
             float mx = -__builtin_inff();
@@ -514,12 +552,12 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             constexpr int K0 = 3 * KC * TWW;
             acc_t acc2[2][KC];
 #pragma unroll
-            for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, K0 + c, &oq[8 * c]);
+            for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, K0 + c, fragments(oq, act, 8 * c));
 #pragma unroll
             for (int i = 0; i < TWW; i++) {
-                if (i + 1 < TWW)
+                if (AHEAD && i + 1 < TWW)
 #pragma unroll
-                    for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, K0 + KC * (i + 1) + c, &oq[8 * c]);
+                    for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, K0 + KC * (i + 1) + c, fragments(oq, act, 8 * c));
                 v4f bo[4];
                 load_tile16(pA + C::A_BOUT + 32 * (t0 + i), g, bo);
                 const float sw = pA[C::A_SW + 3 * TW + t0 + i];
@@ -527,14 +565,17 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int k = 0; k < 4; k++)
-                        x[i][4 * j + k] = x[i][4 * j + k] + (chunk_sum<KC>(acc2[i & 1], 4 * j + k, so) * sw + bo[j][k]);
+                        x[i][4 * j + k] = x[i][4 * j + k] + (chunk_sum<KC>(acc2[AHEAD ? i & 1 : 0], 4 * j + k, so) * sw + bo[j][k]);
                 pin16(x[i]);
                 if (TAPS && a.taps.acc_out)
 #pragma unroll
                     for (int c = 0; c < KC; c++)
 #pragma unroll
                         for (int r = 0; r < 16; r++)
-                            a.taps.acc_out[((bl * KC + c) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = accbits(acc2[i & 1][c], r);
+                            a.taps.acc_out[((bl * KC + c) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = accbits(acc2[AHEAD ? i & 1 : 0][c], r);
+                if (!AHEAD && i + 1 < TWW)
+#pragma unroll
+                    for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, K0 + KC * (i + 1) + c, fragments(oq, act, 8 * c));
             }
         }
         // the attention-phase parameters are dead: fetch the next layer's
@@ -560,12 +601,12 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 float am = 0.0f;
                 acc_t acc2[2][KC];
 #pragma unroll
-                for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + c, &xq[8 * c]);
+                for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + c, fragments(xq, act, 8 * c));
 #pragma unroll
                 for (int i = 0; i < HT; i++) {
-                    if (i + 1 < HT)
+                    if (AHEAD && i + 1 < HT)
 #pragma unroll
-                        for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, k1 + KC * (i + 1) + c, &xq[8 * c]);
+                        for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, k1 + KC * (i + 1) + c, fragments(xq, act, 8 * c));
                     v4f b1[4];
                     load_tile16(pB + C::B_BFF1 + 128 * st + 32 * (h0 + i), g, b1);
                     const float sw = pB[C::B_SW + 4 * st + h0 + i];
@@ -573,7 +614,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                     for (int j = 0; j < 4; j++)
 #pragma unroll
                         for (int k = 0; k < 4; k++) {
-                            const float v = __builtin_fmaxf(chunk_sum<KC>(acc2[i & 1], 4 * j + k, sa) * sw + b1[j][k], 0.0f);
+                            const float v = __builtin_fmaxf(chunk_sum<KC>(acc2[AHEAD ? i & 1 : 0], 4 * j + k, sa) * sw + b1[j][k], 0.0f);
                             hf[i][4 * j + k] = v;
                             am = __builtin_fmaxf(am, v);
                         }
@@ -583,7 +624,10 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                         for (int c = 0; c < KC; c++)
 #pragma unroll
                             for (int r = 0; r < 16; r++)
-                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + ch(r, g)] = accbits(acc2[i & 1][c], r);
+                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + ch(r, g)] = accbits(acc2[AHEAD ? i & 1 : 0][c], r);
+                    if (!AHEAD && i + 1 < HT)
+#pragma unroll
+                        for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + KC * (i + 1) + c, fragments(xq, act, 8 * c));
                 }
                 // quantiser over the 256-wide chunk this wave shares with its neighbour (waves 0,1: first
                 // chunk of the step; 2,3: second).  int8: unsigned, bytes stored as q - 128 for the signed
@@ -621,22 +665,25 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             const int k2 = k1 + HT * KC;
             acc_t acc2[2];
             v4i hqc[8];
+            if constexpr (!ACTL)
 #pragma unroll
-            for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + s * FRAG + lane * 16);
-            acc2[0] = BF_WMM(false, k2, &hqc[0]);
+                for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + s * FRAG + lane * 16);
+            acc2[0] = BF_WMM(false, k2, fragments(hqc, hid, 0));
 #pragma unroll
             for (int idx = 0; idx < 2 * TWW; idx++) {
                 const int c = idx / TWW, i = idx % TWW;
                 v4i ws[4];
                 if (!FP8) load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * (t0 + i), g, ws);
-                if (idx + 1 < 2 * TWW) {
+                if (AHEAD && idx + 1 < 2 * TWW) {
                     if ((idx + 1) % TWW == 0)
 #pragma unroll
                         for (int s = 0; s < 8; s++)
                             hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * (c + 1) + s) * FRAG + lane * 16);
-                    acc2[(idx + 1) & 1] = BF_WMM(false, k2 + idx + 1, &hqc[0]);
+                    acc2[(idx + 1) & 1] = BF_WMM(false, k2 + idx + 1, fragments(hqc, hid, 0));
                 }
-                const acc_t acc = acc2[idx & 1];
+                if (!AHEAD && idx > 0)
+                    acc2[0] = BF_WMM(false, k2 + idx, (FragSrc{&hqc[0], hid + 8 * c * FRAG + lane * 16}));
+                const acc_t acc = acc2[AHEAD ? idx & 1 : 0];
                 if constexpr (FP8) {
                     // descale each 256-deep tile with its own scales, fp32 sum over the tiles
                     const float sw = pB[C::B_SW + 16 + (t0 + i) * KCF + 2 * st + c];

@@ -30,8 +30,8 @@ static bool shape512(const bf_shape* s) {
 static bool board_shape_ok(const bf_shape* s) { return shape_ok(s) || shape512(s); }
 
 // AUTO runs one workgroup per compute unit (lowest latency per position; eight wavefronts per
-// position where that form exists, else four) up to this many positions, which is one per
-// compute unit of an MI355X; above it, two workgroups per compute unit (highest throughput).
+// position in int8, four in e4m3) up to this many positions, which is one per compute unit of an
+// MI355X; above it, two workgroups per compute unit (highest throughput; 256-wide network).
 static const int64_t kBoardMaxN = 256;
 
 template <int DM>
@@ -103,7 +103,7 @@ static int choose_kernel(const bf_eval_args* a) {
     // the board blobs are packed for one format; the 512-wide network runs int8 only
     const bool board_can = have_board && (a->quant == BF_QUANT_INT8 || shape_ok(&a->shape));
     const bool twin_can = have_board && shape_ok(&a->shape);
-    const bool octo_can = twin_can && a->quant == BF_QUANT_INT8;
+    const bool octo_can = have_board && a->quant == BF_QUANT_INT8;   // either width
     switch (a->kernel) {
     case BF_KERNEL_QUAD:
         if (!quad_can) return fail(BF_ERR_UNSUPPORTED, "the four-positions-per-workgroup kernel needs the 256-wide network and wstream/fparams");
@@ -117,7 +117,7 @@ static int choose_kernel(const bf_eval_args* a) {
         return BF_KERNEL_TWIN;
     case BF_KERNEL_OCTO:
         if (!octo_can)
-            return fail(BF_ERR_UNSUPPORTED, "the eight-wavefronts-per-position kernel needs the 256-wide network, board_wstream/board_fparams and the int8 format");
+            return fail(BF_ERR_UNSUPPORTED, "the eight-wavefronts-per-position kernel needs board_wstream/board_fparams and the int8 format");
         return BF_KERNEL_OCTO;
     case BF_KERNEL_AUTO:
         if (board_can) {
@@ -180,7 +180,10 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream
     hipError_t e;
     if (kind == BF_KERNEL_OCTO) {
         if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
-        e = a->taps ? bf::launch_octo256_taps(k, stream) : bf::launch_octo256(k, stream);
+        if (a->shape.d_model == 512)
+            e = a->taps ? bf::launch_octo512_taps(k, stream) : bf::launch_octo512(k, stream);
+        else
+            e = a->taps ? bf::launch_octo256_taps(k, stream) : bf::launch_octo256(k, stream);
     } else if (kind == BF_KERNEL_TWIN) {
         if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
         if (a->quant == BF_QUANT_E4M3)

@@ -500,9 +500,9 @@ class FusedEncoder:
             raise NotImplementedError("the 512-wide network runs in int8 only")
         if fp8 and kernel == "octo":
             raise NotImplementedError("the eight-wavefront kernel runs in int8 only")
-        if wide and kernel in ("quad", "twin", "octo"):
-            raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernel "
-                                      "(kernel='board' or 'auto') only")
+        if wide and kernel in ("quad", "twin"):
+            raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernels "
+                                      "(kernel='octo', 'board' or 'auto') only")
         if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
             raise ValueError("the evaluator implements pre-norm ReLU layers only")
         self.n_value = int(net.value.weight.shape[0]) if net is not None else 1
@@ -565,7 +565,7 @@ class FusedEncoder:
         elif self.board_wstream is None:
             per = names["quad"]
         elif self.d_model != self.D:
-            per = names["board"]
+            per = names["octo"]
         else:
             per = "1 board/workgroup, 1 or 2 workgroups/CU by batch size"
         return f"{fmt} FFN+QKV+out_proj, {per} (gfx950)"

@@ -102,15 +102,17 @@ def test_kernel_choice_follows_shape_blobs_and_batch_size():
     a.kernel, a.quant, a.board_wstream = 0, 0, None                     # no board blobs: always quad
     a.n = 1
     assert lib.bf_kernel_choice(ctypes.byref(a)) == 1
-    a.shape = hip_impl._Shape(512, 16, 16, 2048, 1, 1e-5)               # the 512-wide network: BOARD at any size
+    a.shape = hip_impl._Shape(512, 16, 16, 2048, 1, 1e-5)               # the 512-wide network: OCTO at any size
     a.board_wstream = 16
-    a.n = 100000
-    assert lib.bf_kernel_choice(ctypes.byref(a)) == 2
-    for forced in (1, 3, 4):
+    for n in (1, 100000):
+        a.n = n
+        assert lib.bf_kernel_choice(ctypes.byref(a)) == 4
+    for forced, want in ((1, -2), (2, 2), (3, -2), (4, 4)):
         a.kernel = forced
-        assert lib.bf_kernel_choice(ctypes.byref(a)) == -2
-    a.kernel, a.quant = 2, 1                                            # ... and in int8 only
-    assert lib.bf_kernel_choice(ctypes.byref(a)) == -2
+        assert lib.bf_kernel_choice(ctypes.byref(a)) == want
+    for forced in (0, 2, 4):                                            # ... and in int8 only
+        a.kernel, a.quant = forced, 1
+        assert lib.bf_kernel_choice(ctypes.byref(a)) < 0
     a.quant = 0
     a.kernel = 7
     assert lib.bf_kernel_choice(ctypes.byref(a)) == -1

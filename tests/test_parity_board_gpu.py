@@ -40,7 +40,7 @@ def base():
 @pytest.fixture(scope="module")
 def stress():
     net, sd = _make(512, 16, 16)
-    return net, sd, encoder_impl("hip")(net, int8=True, out_dtype=torch.float32), c_oracle.COracle(sd)
+    return net, sd, {k: encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=k) for k in ("auto", "octo", "board")}, c_oracle.COracle(sd)
 
 
 def _dev(*ts):
@@ -207,9 +207,12 @@ def test_largest_batch_of_the_sweep_is_independent_of_batch_composition(base):
         assert got.shape[0] == 65536 and torch.equal(got, want[od])
 
 
-def test_stress_network_bit_exact_against_the_c_checker_with_every_tap(stress):
-    net, sd, model, co = stress
-    assert model.kernel_choice(16384) == "board" and model.wstream is None
+@pytest.mark.parametrize("kernel", ["auto", "board"])
+def test_stress_network_bit_exact_against_the_c_checker_with_every_tap(stress, kernel):
+    net, sd, models, co = stress
+    model = models[kernel]
+    assert model.kernel_choice(16384) == ("octo" if kernel == "auto" else "board") and model.wstream is None
+    assert models["octo"].kernel_choice(1) == "octo"
     b, c, r, m = positions.random_positions(12, plies=120, seed=31, stamp_queen=True)
     got = model.forward_taps(*_dev(b, c, r), mask=m.cuda())
     want = co.forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy(), taps=True)
@@ -230,7 +233,7 @@ def test_stress_network_bit_exact_against_the_c_checker_with_every_tap(stress):
     p, q2, v = model.forward_full(bd, cd, rd, md)
     assert torch.equal(p, got["policy"]) and torch.equal(q2, got["promo"]) and torch.equal(v, got["value"])
     assert torch.equal(model.best_move, got["best"])
-    half = encoder_impl("hip")(net, int8=True).forward_full(bd, cd, rd, md)[0]
+    half = encoder_impl("hip")(net, int8=True, kernel=kernel).forward_full(bd, cd, rd, md)[0]
     assert half.dtype is torch.float16 and torch.equal(half, p.half())
     x_in = torch.from_numpy(want["resid"][:, 10]).cuda()
     tail = model.forward_taps(bd, cd, rd, mask=md, x_in=x_in, layer_begin=11, layer_end=16, want=["resid"])
@@ -252,6 +255,7 @@ def test_stress_network_win_draw_loss_head_and_full_batch_properties():
     # size-independent properties on everything
     net, sd = _make(512, 16, 16, nv=3, seed=2)
     model = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
+    assert model.kernel_choice(16384) == "octo"
     co = c_oracle.COracle(sd)
     n = 16384
     b, c, r, m = positions.random_positions(n, plies=120, seed=0)
@@ -263,6 +267,11 @@ def test_stress_network_win_draw_loss_head_and_full_batch_properties():
     assert _bits_equal(v[idx], want["value"]) and (best.cpu().numpy()[idx] == want["best"]).all()
     part = model.forward_masked(bd[9000:9700], cd[9000:9700], rd[9000:9700], md[9000:9700])
     assert torch.equal(part[0], p[9000:9700]) and torch.equal(part[3], best[9000:9700])
+    # the four-wavefront form returns the same bits
+    other = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="board")
+    part = other.forward_masked(bd[3000:4100], cd[3000:4100], rd[3000:4100], md[3000:4100])
+    for x, y in zip(part, (p, q, v, best)):
+        assert torch.equal(x, y[3000:4100])
     legal = ((md[..., None] >> torch.arange(64, device="cuda")) & 1).bool()
     assert torch.isneginf(p[~legal]).all() and torch.isfinite(p[legal]).all() and (v.abs() <= 1).all()
     has = legal.reshape(n, -1).any(1)
