@@ -44,18 +44,19 @@ enum bf_quant {
  *   QUAD   four positions per workgroup, one wavefront each, weights shared through LDS; carries
  *          the phase profile (256-wide network, int8 and e4m3).
  *   BOARD  one position per workgroup, the four wavefronts split the model width; one workgroup
- *          per compute unit: low latency per position (launches that cannot fill the GPU) and
- *          the only kernel the 512-wide network fits.
+ *          per compute unit: low latency per position (launches that cannot fill the GPU);
+ *          both network widths.
  *   TWIN   the BOARD decomposition shaped so that two workgroups share a compute unit (each SIMD
  *          holds two wavefronts that cover each other's waits): the highest throughput
  *          (256-wide network).
  *   OCTO   the BOARD decomposition with eight wavefronts per position (two per quarter of the
  *          width, each taking half of the quarter's tiles), one workgroup per compute unit: the
- *          lowest latency per position (256-wide network, int8).
+ *          lowest latency per position for the 256-wide network, and the faster kernel for the
+ *          512-wide one (int8).
  * BOARD, TWIN and OCTO read the same blobs (board_wstream / board_fparams).  The 256-wide network
  * runs in int8 on all four and in e4m3 on QUAD, BOARD and TWIN; the 512-wide network in int8 on
- * BOARD.  For the 256-wide network the kernels return bit-identical results in either format, so
- * AUTO may pick by batch size. */
+ * OCTO and BOARD.  Kernels that carry a network and a format return bit-identical results for
+ * it, so AUTO may pick by batch size. */
 enum bf_kernel {
     BF_KERNEL_AUTO = 0,
     BF_KERNEL_QUAD = 1,
@@ -157,8 +158,8 @@ typedef struct {
      * QUAD: the wavefront runs on, storing nothing) */
     const uint8_t* active;
     int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: for n <= bf_board_max_n()
-                             * OCTO (int8, 256-wide network) or BOARD (e4m3; the 512-wide
-                             * network at any n), TWIN above; without them QUAD */
+                             * OCTO (int8) or BOARD (e4m3), TWIN above; the 512-wide
+                             * network: OCTO at any n; without the board blobs QUAD */
 } bf_eval_args;
 
 /* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */
