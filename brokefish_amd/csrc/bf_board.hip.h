@@ -38,9 +38,10 @@
 
 // TWIN form: workgroups per compute unit, and register sets of the weight prefetch (one set =
 // half a block; SETS - 1 half-blocks are in flight).  Measured on MI355X at batch 4096: three
-// workgroups per unit spill too much (1.42 M evals/s against 2.10 M), four sets beat three by 2 %.
+// workgroups per unit spill too much (81-103 registers); three sets run without a spill
+// (1.717 ms), four spill 8 registers (1.741 ms), six 61 (2.10 ms).
 #ifndef BF_TWIN_SETS
-#define BF_TWIN_SETS 4
+#define BF_TWIN_SETS 3
 #endif
 #ifndef BF_TWIN_OCC
 #define BF_TWIN_OCC 2
@@ -167,9 +168,13 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     // Eight wavefronts on the 512-wide network: a wave has 256 registers and the quantised row alone
     // would take 64 of them, so the activation fragments are read from LDS at each MFMA instead.
     constexpr bool ACTL = OCTO && DM == 512;
-    // ... and the next tile's product is issued after a tile's epilogue, not before it (one set of
-    // accumulators instead of two; the SIMD's other wave fills the gap)
-    constexpr bool AHEAD = !ACTL;
+    // One wave per SIMD (!TWIN, 512 registers): a tile's product is issued before the previous
+    // tile's epilogue, and Q, K and V together, so the matrix pipe works under the vector work of
+    // the same wave.  Two waves per SIMD (256 registers each): one product at a time, issued after
+    // the previous epilogue -- the second set of accumulators would spill, and the SIMD's other
+    // wave fills the gap.  Measured at batch 4096 (TWIN): 1.72 ms without a spill, against
+    // 1.90 ms with 20 spilled registers when issuing ahead.
+    constexpr bool AHEAD = !TWIN;
     constexpr int HALF = BLOCK / 2;   // four fragments: the unit of the register prefetch (TWIN)
     constexpr int VM_AHEAD = TAPS ? 0 : (SLOTS - 1) * 8;   // ring loads that may stay in flight at a ring wait
     const int lane = threadIdx.x & 63;
@@ -451,7 +456,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         acc_t accq[KC], acck[KC], accv[KC];
 #pragma unroll
         for (int i = 0; i < TWW; i++) {
-            if (AHEAD && (TWIN || i == 0)) {
+            if (AHEAD && i == 0) {
 #pragma unroll
                 for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * i + c, fragments(xq, act, 8 * c));
 #pragma unroll
@@ -512,7 +517,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             v16f sc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
             for (int r = 0; r < 16; r++) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[r], qf[r], sc, 0, 0, 0);
-            if (!TWIN && i + 1 < TWW) {
+            if (AHEAD && i + 1 < TWW) {
 #pragma unroll
                 for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * (i + 1) + c, fragments(xq, act, 8 * c));
 #pragma unroll
@@ -681,8 +686,13 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                             hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * (c + 1) + s) * FRAG + lane * 16);
                     acc2[(idx + 1) & 1] = BF_WMM(false, k2 + idx + 1, fragments(hqc, hid, 0));
                 }
-                if (!AHEAD && idx > 0)
+                if (!AHEAD && idx > 0) {
+                    if (!ACTL && idx % TWW == 0)   // the next chunk of the hidden row
+#pragma unroll
+                        for (int s = 0; s < 8; s++)
+                            hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * c + s) * FRAG + lane * 16);
                     acc2[0] = BF_WMM(false, k2 + idx, (FragSrc{&hqc[0], hid + 8 * c * FRAG + lane * 16}));
+                }
                 const acc_t acc = acc2[AHEAD ? idx & 1 : 0];
                 if constexpr (FP8) {
                     // descale each 256-deep tile with its own scales, fp32 sum over the tiles
