@@ -28,7 +28,7 @@ PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s
 PEAK_FP16_OPS = 2.5e15                # dense fp16 MFMA: the e4m3 format's products run on the fp16 instruction
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/
 # (calibrated on a 1 GiB copy), by (network shape, kernel, batch).
-MEASURED_TRAFFIC_BYTES = {("base", "twin", 4096): 1.00e9, ("base", "quad", 4096): 3.07e9,
+MEASURED_TRAFFIC_BYTES = {("base", "twin", 4096): 0.81e9, ("base", "quad", 4096): 3.07e9,
                           ("base", "board", 256): 5.5e7, ("base", "octo", 256): 5.5e7, ("stress", "board", 16384): 2.66e10,
                           ("stress", "octo", 16384): 3.36e10}
 MEASURED_TRAFFIC_BYTES_E4M3 = {("base", "twin", 4096): 0.97e9}
