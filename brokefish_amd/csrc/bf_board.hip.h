@@ -46,16 +46,11 @@
 #ifndef BF_TWIN_OCC
 #define BF_TWIN_OCC 2
 #endif
-// Eight-wavefront form: one workgroup per compute unit leaves each wave 256 registers of which the
-// kernel needs fewer, and a launch that small is bound by the latency of the weight stream, not
-// by its bandwidth: more half-blocks in flight.
+// Eight-wavefront form: register sets of its weight prefetch.  Measured: 256-wide network, 64
+// positions: 0.136 ms with four sets, 0.137 with three, 0.138 with six; 512-wide network, 4096
+// positions: 12.5 ms with four, 12.8 with three, 16.0 with six (68 spilled registers).
 #ifndef BF_OCTO_SETS
-#define BF_OCTO_SETS 6
-#endif
-// ... on the 512-wide network the form runs whole batches and registers are scarce: four sets
-// (measured at 4096 positions: 12.5 ms; three sets 12.8, six 16.0)
-#ifndef BF_OCTO_SETS_WIDE
-#define BF_OCTO_SETS_WIDE 4
+#define BF_OCTO_SETS 4
 #endif
 
 namespace bf {
@@ -162,7 +157,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     constexpr int HT = 4 / SUB;               // hidden tiles a wave computes per feed-forward step
     constexpr int NB = BPW / SUB;             // weight blocks a wave consumes per layer
     // register sets of the prefetch: NSETS - 1 half-blocks in flight
-    constexpr int NSETS = !OCTO ? BF_TWIN_SETS : DM == 256 ? BF_OCTO_SETS : BF_OCTO_SETS_WIDE;
+    constexpr int NSETS = OCTO ? BF_OCTO_SETS : BF_TWIN_SETS;
     static_assert(TW % SUB == 0 && (2 * NB) % NSETS == 0, "tiles and register sets must split evenly");
     constexpr int XS = NW * 64;               // floats of one exchange slot
     // Eight wavefronts on the 512-wide network: a wave has 256 registers and the quantised row alone
