@@ -407,10 +407,11 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         // !TWIN: the block is in `fr`; the ring slot it came from is refilled SLOTS blocks ahead,
         // then block k+1 is read from its slot.
         const int lbase = li * BPW, lfollow = OCTO ? (lnext - a.l0) * BPW : (li + 1) * BPW;
-#define BF_WMM(SWAP, k, actp)                                                                        \
+#define BF_WMM(SWAP, k, actp) BF_WMM_FROM(SWAP, k, actp, (acc_t{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}))
+#define BF_WMM_FROM(SWAP, k, actp, init)                                                             \
     ([&]() -> acc_t {                                                                                \
         const FragSrc act_ = (actp);                                                                 \
-        acc_t r_ = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};                                 \
+        acc_t r_ = (init);                                                                           \
         if constexpr (TWIN) {                                                                        \
             fetch_half(2 * (k) + NSETS - 1, lbase, lfollow);                                         \
             _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++)                                         \
@@ -668,12 +669,27 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             if constexpr (!ACTL)
 #pragma unroll
                 for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + s * FRAG + lane * 16);
-            acc2[0] = BF_WMM(false, k2, fragments(hqc, hid, 0));
+            // int8, one product at a time: the accumulator starts at 128 * sum(w) (the offset of the
+            // unsigned operand bytes stored as q - 128), which saves adding it afterwards
+            constexpr bool WFOLD = !AHEAD && !FP8;
+            auto wsum_start = [&](int idx) -> acc_t {
+                acc_t r = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                if constexpr (WFOLD) {
+                    v4i w0[4];
+                    load_tile16i(pB + C::B_WSUM + (2 * st + idx / TWW) * CW + 32 * (t0 + idx % TWW), g, w0);
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int k = 0; k < 4; k++) r[4 * j + k] = w0[j][k];
+                }
+                return r;
+            };
+            acc2[0] = BF_WMM_FROM(false, k2, fragments(hqc, hid, 0), wsum_start(0));
 #pragma unroll
             for (int idx = 0; idx < 2 * TWW; idx++) {
                 const int c = idx / TWW, i = idx % TWW;
-                v4i ws[4];
-                if (!FP8) load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * (t0 + i), g, ws);
+                v4i ws[4] = {};
+                if (!FP8 && !WFOLD) load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * (t0 + i), g, ws);
                 if (AHEAD && idx + 1 < 2 * TWW) {
                     if ((idx + 1) % TWW == 0)
 #pragma unroll
@@ -686,7 +702,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
                         for (int s = 0; s < 8; s++)
                             hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * c + s) * FRAG + lane * 16);
-                    acc2[0] = BF_WMM(false, k2 + idx, (FragSrc{&hqc[0], hid + 8 * c * FRAG + lane * 16}));
+                    acc2[0] = BF_WMM_FROM(false, k2 + idx, (FragSrc{&hqc[0], hid + 8 * c * FRAG + lane * 16}), wsum_start(idx));
                 }
                 const acc_t acc = acc2[AHEAD ? idx & 1 : 0];
                 if constexpr (FP8) {
@@ -706,7 +722,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                     for (int j = 0; j < 4; j++)
 #pragma unroll
                         for (int k = 0; k < 4; k++) {
-                            const int full = accbits(acc, 4 * j + k) + ws[j][k];
+                            const int full = WFOLD ? accbits(acc, 4 * j + k) : accbits(acc, 4 * j + k) + ws[j][k];
                             o64[i][4 * j + k] = (st == 0 && c == 0) ? (double)full * sc
                                                                     : __builtin_fma((double)full, sc, o64[i][4 * j + k]);
                             if (TAPS && a.taps.acc_ff2)
@@ -735,6 +751,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         dma(wpar + (size_t)lnext * C::PW_FLOATS + C::A_FLOATS, pB, C::B_FLOATS, lane);
 #undef BF_WMM
+#undef BF_WMM_FROM
         if (TAPS && a.taps.resid)
 #pragma unroll
             for (int i = 0; i < TWW; i++)
