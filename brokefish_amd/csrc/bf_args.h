@@ -139,10 +139,12 @@ hipError_t launch_twin256_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_twin256_fp8(const KArgs& k, hipStream_t stream);
 hipError_t launch_twin256_fp8_taps(const KArgs& k, hipStream_t stream);
 // one position per workgroup of eight wavefronts (two per quarter of the width), one workgroup
-// per compute unit, int8: the lowest latency per position for the 256-wide network, and the
-// faster form for the 512-wide one
+// per compute unit: the lowest latency per position for the 256-wide network (int8, e4m3), and
+// the faster form for the 512-wide one (int8)
 hipError_t launch_octo256(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo256_taps(const KArgs& k, hipStream_t stream);
+hipError_t launch_octo256_fp8(const KArgs& k, hipStream_t stream);
+hipError_t launch_octo256_fp8_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512_taps(const KArgs& k, hipStream_t stream);
 

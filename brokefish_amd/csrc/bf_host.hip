@@ -29,9 +29,9 @@ static bool shape512(const bf_shape* s) {
 
 static bool board_shape_ok(const bf_shape* s) { return shape_ok(s) || shape512(s); }
 
-// AUTO runs one workgroup per compute unit (lowest latency per position; eight wavefronts per
-// position in int8, four in e4m3) up to this many positions, which is one per compute unit of an
-// MI355X; above it, two workgroups per compute unit (highest throughput; 256-wide network).
+// AUTO runs one workgroup of eight wavefronts per compute unit (lowest latency per position) up
+// to this many positions, which is one per compute unit of an MI355X; above it, two workgroups
+// of four wavefronts per compute unit (highest throughput; 256-wide network).
 static const int64_t kBoardMaxN = 256;
 
 template <int DM>
@@ -103,7 +103,7 @@ static int choose_kernel(const bf_eval_args* a) {
     // the board blobs are packed for one format; the 512-wide network runs int8 only
     const bool board_can = have_board && (a->quant == BF_QUANT_INT8 || shape_ok(&a->shape));
     const bool twin_can = have_board && shape_ok(&a->shape);
-    const bool octo_can = have_board && a->quant == BF_QUANT_INT8;   // either width
+    const bool octo_can = board_can;   // the same networks and formats as BOARD
     switch (a->kernel) {
     case BF_KERNEL_QUAD:
         if (!quad_can) return fail(BF_ERR_UNSUPPORTED, "the four-positions-per-workgroup kernel needs the 256-wide network and wstream/fparams");
@@ -117,13 +117,10 @@ static int choose_kernel(const bf_eval_args* a) {
         return BF_KERNEL_TWIN;
     case BF_KERNEL_OCTO:
         if (!octo_can)
-            return fail(BF_ERR_UNSUPPORTED, "the eight-wavefronts-per-position kernel needs board_wstream/board_fparams and the int8 format");
+            return fail(BF_ERR_UNSUPPORTED, "the eight-wavefronts-per-position kernel needs board_wstream/board_fparams (512-wide network: the int8 format)");
         return BF_KERNEL_OCTO;
     case BF_KERNEL_AUTO:
-        if (board_can) {
-            if (twin_can && a->n > kBoardMaxN) return BF_KERNEL_TWIN;
-            return octo_can ? BF_KERNEL_OCTO : BF_KERNEL_BOARD;
-        }
+        if (octo_can) return (twin_can && a->n > kBoardMaxN) ? BF_KERNEL_TWIN : BF_KERNEL_OCTO;
         if (quad_can) return BF_KERNEL_QUAD;
         return fail(BF_ERR_ARGUMENT, shape512(&a->shape)
                         ? "the 512-wide network runs on the one-position-per-workgroup kernel: int8, board_wstream/board_fparams required"
@@ -182,6 +179,8 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream
         if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
         if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_octo512_taps(k, stream) : bf::launch_octo512(k, stream);
+        else if (a->quant == BF_QUANT_E4M3)
+            e = a->taps ? bf::launch_octo256_fp8_taps(k, stream) : bf::launch_octo256_fp8(k, stream);
         else
             e = a->taps ? bf::launch_octo256_taps(k, stream) : bf::launch_octo256(k, stream);
     } else if (kind == BF_KERNEL_TWIN) {

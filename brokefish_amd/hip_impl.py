@@ -498,8 +498,6 @@ class FusedEncoder:
         wide = self.d_model != self.D
         if wide and fp8:
             raise NotImplementedError("the 512-wide network runs in int8 only")
-        if fp8 and kernel == "octo":
-            raise NotImplementedError("the eight-wavefront kernel runs in int8 only")
         if wide and kernel in ("quad", "twin"):
             raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernels "
                                       "(kernel='octo', 'board' or 'auto') only")

@@ -52,11 +52,11 @@ enum bf_quant {
  *   OCTO   the BOARD decomposition with eight wavefronts per position (two per quarter of the
  *          width, each taking half of the quarter's tiles), one workgroup per compute unit: the
  *          lowest latency per position for the 256-wide network, and the faster kernel for the
- *          512-wide one (int8).
+ *          512-wide one.
  * BOARD, TWIN and OCTO read the same blobs (board_wstream / board_fparams).  The 256-wide network
- * runs in int8 on all four and in e4m3 on QUAD, BOARD and TWIN; the 512-wide network in int8 on
- * OCTO and BOARD.  Kernels that carry a network and a format return bit-identical results for
- * it, so AUTO may pick by batch size. */
+ * runs in int8 and e4m3 on all four; the 512-wide network in int8 on OCTO and BOARD.  Kernels that
+ * carry a network and a format return bit-identical results for it, so AUTO may pick by batch
+ * size. */
 enum bf_kernel {
     BF_KERNEL_AUTO = 0,
     BF_KERNEL_QUAD = 1,
@@ -157,9 +157,9 @@ typedef struct {
      * paying for the leaves that need no evaluation (BOARD / TWIN: the workgroup exits at once;
      * QUAD: the wavefront runs on, storing nothing) */
     const uint8_t* active;
-    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: for n <= bf_board_max_n()
-                             * OCTO (int8) or BOARD (e4m3), TWIN above; the 512-wide
-                             * network: OCTO at any n; without the board blobs QUAD */
+    int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: OCTO for
+                             * n <= bf_board_max_n() and for the 512-wide network, TWIN
+                             * above; without the board blobs QUAD */
 } bf_eval_args;
 
 /* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */

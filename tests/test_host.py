@@ -92,13 +92,13 @@ def test_kernel_choice_follows_shape_blobs_and_batch_size():
     for forced in (1, 2, 3, 4):
         a.n, a.kernel = 4096, forced
         assert lib.bf_kernel_choice(ctypes.byref(a)) == forced
-    a.kernel, a.quant = 0, 1                                            # e4m3: BOARD up to the cut
-    for n, want in ((1, 2), (cut, 2), (cut + 1, 3), (4096, 3)):
+    a.kernel, a.quant = 0, 1                                            # e4m3: the same rule
+    for n, want in ((1, 4), (cut, 4), (cut + 1, 3), (4096, 3)):
         a.n = n
         assert lib.bf_kernel_choice(ctypes.byref(a)) == want
-    for forced, want in ((1, 1), (2, 2), (3, 3), (4, -2)):
+    for forced in (1, 2, 3, 4):
         a.kernel = forced
-        assert lib.bf_kernel_choice(ctypes.byref(a)) == want
+        assert lib.bf_kernel_choice(ctypes.byref(a)) == forced
     a.kernel, a.quant, a.board_wstream = 0, 0, None                     # no board blobs: always quad
     a.n = 1
     assert lib.bf_kernel_choice(ctypes.byref(a)) == 1

@@ -114,7 +114,7 @@ def test_automatic_choice_switches_kernel_by_batch_size_without_changing_results
     for x, y in zip(big, ref):
         assert torch.equal(x, y)
     fp8 = encoder_impl("hip")(net, fp8=True)                                             # the same rule in e4m3
-    assert fp8.kernel_choice(1) == "board" and fp8.kernel_choice(cut) == "board" and fp8.kernel_choice(4096) == "twin"
+    assert fp8.kernel_choice(1) == "octo" and fp8.kernel_choice(cut) == "octo" and fp8.kernel_choice(4096) == "twin"
 
 
 def test_e4m3_on_the_throughput_kernel_equals_the_four_per_workgroup_kernel(base):
@@ -136,15 +136,16 @@ def test_e4m3_on_the_throughput_kernel_equals_the_four_per_workgroup_kernel(base
         assert tt[k].dtype == tq[k].dtype and torch.equal(tt[k].view(torch.uint8), tq[k].view(torch.uint8)), k
     int8 = boards["twin"].forward_full(bd, cd, rd)[0]
     assert not torch.equal(int8, twin.forward_full(bd, cd, rd)[0])
-    # the one-workgroup-per-compute-unit kernel carries the format too, and AUTO switches by size
-    board = encoder_impl("hip")(net, fp8=True, out_dtype=torch.float32, kernel="board")
-    for x, y in zip(board.forward_masked(bd, cd, rd, md), got):
-        assert torch.equal(x, y)
-    tb = board.forward_taps(bd[:40], cd[:40], rd[:40])
-    for k in TAPS:
-        assert torch.equal(tb[k].view(torch.uint8), tq[k].view(torch.uint8)), k
+    # the one-workgroup-per-compute-unit kernels carry the format too, and AUTO switches by size
+    for kernel in ("board", "octo"):
+        other = encoder_impl("hip")(net, fp8=True, out_dtype=torch.float32, kernel=kernel)
+        for x, y in zip(other.forward_masked(bd, cd, rd, md), got):
+            assert torch.equal(x, y), kernel
+        tb = other.forward_taps(bd[:40], cd[:40], rd[:40])
+        for k in TAPS:
+            assert torch.equal(tb[k].view(torch.uint8), tq[k].view(torch.uint8)), (kernel, k)
     auto = encoder_impl("hip")(net, fp8=True, out_dtype=torch.float32)
-    assert auto.kernel_choice(256) == "board" and auto.kernel_choice(257) == "twin"
+    assert auto.kernel_choice(256) == "octo" and auto.kernel_choice(257) == "twin"
     small = [t.clone() for t in auto.forward_masked(bd[:200], cd[:200], rd[:200], md[:200])]
     for x, y in zip(small, got):
         assert torch.equal(x, y[:200])
