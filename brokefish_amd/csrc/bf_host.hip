@@ -3,6 +3,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "bf_args.h"
 
@@ -216,6 +217,64 @@ extern "C" int bf_model_forward(const bf_eval_args* args, void* stream) {
     const int rc = check_args(args, &k, &kind);
     if (rc) return rc;
     return launch(args, k, kind, (hipStream_t)stream);
+}
+
+// ---- the entry point that allocates nothing ----------------------------------------------------
+// The four-positions-per-workgroup kernel parks the residual stream in a workspace the caller
+// lends to bf_model_forward.  For callers that cannot allocate, the same launch with the
+// workspace in this file-scope device array.  Each GPU the library runs on holds its own copy
+// at its own address until the process ends; `scratch` is the host-side stand-in of the symbol
+// and is never passed to a kernel: host code uses the per-device address looked up below.
+static __device__ __align__(256) uint8_t scratch[(size_t)BF_STATIC_MAX_N * bf::T * bf::D * sizeof(float)];
+
+static const int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices];   // device address of `scratch` on device i, NULL until looked up
+
+// The address of this device's copy of `scratch`, looked up once per device with that device
+// current (the caller's current device is the one the launch goes to).
+static int scratch_address(void** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(BF_ERR_DEVICE, "no current HIP device (or its ordinal is 64 or more)");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            snprintf(g_err, sizeof(g_err), "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+            return BF_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return BF_OK;
+}
+
+extern "C" int bf_model_forward_static(const bf_eval_args* args, void* stream) {
+    if (!args) return fail(BF_ERR_ARGUMENT, "args is NULL");
+    if (args->kernel != BF_KERNEL_AUTO && args->kernel != BF_KERNEL_QUAD)
+        return fail(BF_ERR_ARGUMENT, "bf_model_forward_static runs the four-positions-per-workgroup kernel: kernel must be BF_KERNEL_QUAD "
+                                     "or BF_KERNEL_AUTO (the other kernels need no workspace: call bf_model_forward)");
+    if (args->n > BF_STATIC_MAX_N) {
+        snprintf(g_err, sizeof(g_err), "n = %lld exceeds BF_STATIC_MAX_N = %d positions, the size of the library's static workspace",
+                 (long long)args->n, BF_STATIC_MAX_N);
+        return BF_ERR_ARGUMENT;
+    }
+    // the argument checks come first (they touch no device); the placeholder only has to pass them
+    bf_eval_args a = *args;
+    a.kernel = BF_KERNEL_QUAD;
+    a.workspace = reinterpret_cast<void*>(uintptr_t(256));
+    a.workspace_bytes = sizeof(scratch);
+    bf::KArgs k;
+    int kind;
+    const int rc = check_args(&a, &k, &kind);
+    if (rc) return rc;
+    void* ws = nullptr;
+    const int rc0 = scratch_address(&ws);
+    if (rc0) return rc0;
+    k.xpark = static_cast<float*>(ws);
+    return launch(&a, k, kind, (hipStream_t)stream);
 }
 
 extern "C" int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_t* cycles) {

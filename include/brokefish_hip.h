@@ -172,6 +172,20 @@ int bf_kernel_choice(const bf_eval_args* args);
  * brokefish/nn/cuda_impl.py:497-503).  `stream` is a hipStream_t (NULL = default). */
 int bf_model_forward(const bf_eval_args* args, void* stream);
 
+/* The evaluator for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and results as bf_model_forward on the QUAD kernel (args->kernel must be
+ * BF_KERNEL_QUAD or BF_KERNEL_AUTO; wstream / fparams required), except that args->workspace and
+ * args->workspace_bytes are ignored: the kernel's workspace is a static device array of
+ * BF_STATIC_MAX_N * 32 KiB inside the library, which every GPU the library runs on holds until
+ * the process ends.  n above BF_STATIC_MAX_N is rejected with BF_ERR_ARGUMENT.  The call makes
+ * no hipMalloc / hipFree; its first call on a device looks the array's address up (so make one
+ * call per device before capturing).  All calls on one GPU share that GPU's array: calls that
+ * may overlap on one GPU (two streams, two threads) race -- serialise them or use
+ * bf_model_forward with separate workspaces.  Nothing in the array has to start at zero. */
+#define BF_STATIC_MAX_N 1024
+int bf_model_forward_static(const bf_eval_args* args, void* stream);
+
 /* Quantisation maxima of the signed / unsigned activation formats, for the host to pin
  * against its own constants.  Replaces int8_q_max (reference csrc/encoder.cu:1926-1929). */
 void bf_int8_q_max(double* s8, double* u8);

@@ -25,6 +25,10 @@ int main(void) {
     args.n = 16;
     if (bf_model_forward(&args, NULL) != BF_ERR_ARGUMENT || strlen(bf_last_error()) == 0) return 5;
     if (bf_model_forward(NULL, NULL) != BF_ERR_ARGUMENT) return 6;
+    if (bf_model_forward_static(&args, NULL) >= 0 || bf_model_forward_static(NULL, NULL) != BF_ERR_ARGUMENT) return 15;   /* no parameter blobs */
+    args.n = BF_STATIC_MAX_N + 1;
+    if (bf_model_forward_static(&args, NULL) != BF_ERR_ARGUMENT || !strstr(bf_last_error(), "BF_STATIC_MAX_N")) return 16;
+    args.n = 16;
     if (bf_kernel_choice(&args) >= 0) return 7;                 /* no parameter blobs */
     if (bf_time_kernel_ms(&args, NULL, 1, 1) >= 0.0) return 8;
     if (bf_profile_phases(&args, NULL, NULL) >= 0) return 9;
