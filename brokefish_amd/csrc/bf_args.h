@@ -84,8 +84,10 @@ struct Layout {
     static constexpr int SLOTS = DM == 256 ? 3 : 2;  // depth of a wave's private LDS weight ring, in blocks
     static constexpr int A_LN1G = 0, A_LN1B = CW, A_BQ = 2 * CW, A_BK = 3 * CW, A_BV = 4 * CW, A_BOUT = 5 * CW,
                          A_SW = 6 * CW, A_FLOATS = 6 * CW + 16;
-    static constexpr int B_LN2G = 0, B_LN2B = CW, B_BFF1 = 2 * CW, B_BFF2 = 2 * CW + 128 * STEPS,
-                         B_WSUM = 3 * CW + 128 * STEPS, B_SW = B_WSUM + KCF * CW, B_FLOATS = B_SW + 32;
+    // part B: the first B_LDS_FLOATS are read many times per layer; the tail (first feed-forward
+    // bias, 128 * sum(w)) is read once per tile and may be taken from global memory instead of LDS
+    static constexpr int B_LN2G = 0, B_LN2B = CW, B_BFF2 = 2 * CW, B_SW = 3 * CW, B_LDS_FLOATS = 3 * CW + 32,
+                         B_BFF1 = B_LDS_FLOATS, B_WSUM = B_BFF1 + 128 * STEPS, B_FLOATS = B_WSUM + KCF * CW;
     static constexpr int PW_FLOATS = A_FLOATS + B_FLOATS;
     static constexpr int G_SQ = 0, G_TS = 64 * D, G_CT = G_TS + 12 * D, G_CLOCK = G_CT + 4 * D,
                          G_REP = G_CLOCK + 101 * D, G_NFG = G_REP + 3 * D, G_NFB = G_NFG + D,
@@ -147,5 +149,9 @@ hipError_t launch_octo256_fp8(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo256_fp8_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512_taps(const KArgs& k, hipStream_t stream);
+// the int8 builds that carry the phase profile
+hipError_t launch_twin256_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_octo256_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_octo512_prof(const KArgs& k, hipStream_t stream);
 
 }  // namespace bf

@@ -30,9 +30,12 @@
 //                 per position (launches of up to one position per compute unit).
 //
 // LDS map (bytes): [ring: 4 waves x SLOTS x 8 KiB, absent in the TWIN form] [xch: 3 slots of
-// 64 floats per wave] [hid: 16 KiB] [act: NT KiB] [par: PW floats per wave].  During the heads the
+// 64 floats per wave] [hid: 32 KiB (width 256: the whole hidden row) or 16 KiB (width 512: one
+// step)] [act: NT KiB] [par: PW floats per wave].  During the heads the
 // normalised stream (NT*4 KiB, fp32) overlays hid/act/par.
 #pragma once
+
+#include <atomic>
 
 #include "bf_device.hip.h"
 
@@ -49,8 +52,23 @@
 // Eight-wavefront form: register sets of its weight prefetch.  Measured: 256-wide network, 64
 // positions: 0.136 ms with four sets, 0.137 with three, 0.138 with six; 512-wide network, 4096
 // positions: 12.5 ms with four, 12.8 with three, 16.0 with six (68 spilled registers).
+#ifndef BF_TWIN_AHEAD_FFN
+#define BF_TWIN_AHEAD_FFN 1
+#endif
+#ifndef BF_BIASED_ACC
+#define BF_BIASED_ACC 1
+#endif
+#ifndef BF_FORCE_ACTL
+#define BF_FORCE_ACTL 0
+#endif
 #ifndef BF_OCTO_SETS
 #define BF_OCTO_SETS 4
+#endif
+
+#ifdef BF_EXP_NOF32   // timing experiment: one vector instruction in place of an fp32 matrix step
+#define BF_F32MMA(a_, b_, c_) ([&]() { v16f r_ = (c_); r_[0] = __builtin_fmaf((a_), (b_), r_[0]); return r_; }())
+#else
+#define BF_F32MMA(a_, b_, c_) __builtin_amdgcn_mfma_f32_32x32x2f32((a_), (b_), (c_), 0, 0, 0)
 #endif
 
 namespace bf {
@@ -65,9 +83,17 @@ struct Cfg : Layout<DM> {
     static constexpr int RING_BYTES = TWIN ? 0 : 4 * L::SLOTS * BLOCK;
     static constexpr int XCH_OFF = RING_BYTES;
     static constexpr int HID_OFF = XCH_OFF + 3 * (NW / 4) * FRAG;
-    static constexpr int ACT_OFF = HID_OFF + 16 * FRAG;
+    // the quantised hidden row of the feed-forward block: the whole row (32 tiles) for the 256-wide
+    // network, one step of 512 channels (16 tiles) for the 512-wide one, whose row does not fit
+    static constexpr bool FULLHID = DM == 256;
+    static constexpr int HID_FRAGS = FULLHID ? L::F / 32 : 16;
+    static constexpr int ACT_OFF = HID_OFF + HID_FRAGS * FRAG;
     static constexpr int PAR_OFF = ACT_OFF + L::NT * FRAG;
-    static constexpr int LDS_BYTES = PAR_OFF + NW * L::PW_FLOATS * 4;
+    // three workgroups per compute unit: only the often-read part of the feed-forward parameters
+    // is kept in LDS, the rest is read from global memory where it is used
+    static constexpr bool BTAIL_GLOBAL = TWIN && !OCTO && BF_TWIN_OCC >= 3;
+    static constexpr int PWL_FLOATS = L::A_FLOATS + (BTAIL_GLOBAL ? L::B_LDS_FLOATS : L::B_FLOATS);   // per wave, in LDS
+    static constexpr int LDS_BYTES = PAR_OFF + NW * PWL_FLOATS * 4;
     static_assert(!OCTO || TWIN, "eight wavefronts per position take their weights straight to registers");
     static_assert(LDS_BYTES <= (TWIN && !OCTO ? 160 / BF_TWIN_OCC : 160) * 1024, "LDS budget: one or two workgroups per compute unit");
     static_assert(L::NT * 4 * FRAG <= LDS_BYTES - HID_OFF, "normalised stream overlay");
@@ -104,6 +130,11 @@ __device__ __forceinline__ void dma(const float* src, float* dst, int nfloats, i
 // one 16-byte fragment step of a block product: a 32-deep int8 MFMA, or two 16-deep e4m3 steps
 template <bool SWAP>
 __device__ __forceinline__ v16i frag_mma(const v4i& w, const v4i& act, const v16i& acc) {
+#ifdef BF_EXP_NOMFMA   // timing experiment: one vector instruction in place of the product
+    v16i r = acc;
+    r[0] += w[0] ^ act[0];
+    return r;
+#endif
     return SWAP ? __builtin_amdgcn_mfma_i32_32x32x32_i8(act, w, acc, 0, 0, 0)
                 : __builtin_amdgcn_mfma_i32_32x32x32_i8(w, act, acc, 0, 0, 0);
 }
@@ -116,36 +147,75 @@ __device__ __forceinline__ v16f frag_mma(const v4i& w, const v4i& act, v16f acc)
 }
 
 // acc * sa summed over the k-chunks in float64, cast once (one chunk: the fp32 product, which
-// is the same number)
-template <int KC, typename ACC>
+// is the same number).  BIASED: the int32 accumulator started at the bit pattern of 1.5 * 2^23,
+// so its bits read as a float are 1.5 * 2^23 + acc exactly (|acc| <= 127 * 127 * 256 < 2^22) and
+// one fp32 subtraction, which is exact, replaces the slower integer-to-float conversion.
+constexpr int ACC_BIAS_BITS = 0x4b400000;
+constexpr float ACC_BIAS = 12582912.0f;
+template <int KC, bool BIASED, typename ACC>
 __device__ __forceinline__ float chunk_sum(const ACC (&acc)[KC], int i, const float (&sa)[KC]) {
     if constexpr (KC == 1) {
-        return accf(acc[0], i) * sa[0];
+        if constexpr (BIASED) return (__int_as_float(acc[0][i]) - ACC_BIAS) * sa[0];
+        else return accf(acc[0], i) * sa[0];
     } else {
+        static_assert(!BIASED, "the biased accumulator is used with a single k-chunk");
         double o = (double)acc[0][i] * (double)sa[0];
 #pragma unroll
         for (int c = 1; c < KC; c++) o = __builtin_fma((double)acc[c][i], (double)sa[c], o);
         return (float)o;
     }
 }
+// the accumulator's value as the debug taps report it
+template <bool BIASED>
+__device__ __forceinline__ int tapbits(const v16i& a, int i) { return BIASED ? a[i] - ACC_BIAS_BITS : a[i]; }
+template <bool BIASED>
+__device__ __forceinline__ int tapbits(const v16f& a, int i) { return __float_as_int(a[i]); }
 
 // Position of a wave's n-th weight block of a layer inside its quarter's stream: a + sub * b.
 // With four wavefronts per position a wave consumes its quarter's stream in order (a = n).  With
 // eight, the two wavefronts of a quarter (sub = 0, 1) each take half of the quarter's tiles in
 // every matmul, so a wave's blocks are every other group of the same stream.
 struct BlockAt { int a, b; };
-template <int KC, int TW, int SUB>
+template <int KC, int TW, int SUB, bool FULLHID>
 __host__ __device__ constexpr BlockAt block_at(int n) {
     constexpr int TWW = TW / SUB, HT = 4 / SUB;
-    constexpr int NQ = 3 * KC * TWW, NO = KC * TWW, SW_ = HT * KC + 2 * TWW;
+    constexpr int NQ = 3 * KC * TWW, NO = KC * TWW, SSTR = 4 * KC + 2 * TW, BASE = 4 * KC * TW;
     if (n < NQ) return {3 * KC * (n / (3 * KC)) + n % (3 * KC), 3 * KC * TWW};
     if (n < NQ + NO) return {3 * KC * TW + KC * ((n - NQ) / KC) + (n - NQ) % KC, KC * TWW};
-    const int m = n - NQ - NO, st = m / SW_, r = m % SW_, base = 4 * KC * TW + st * (4 * KC + 2 * TW);
-    if (r < HT * KC) return {base + KC * (r / KC) + r % KC, KC * HT};
-    return {base + 4 * KC + ((r - HT * KC) / TWW) * TW + (r - HT * KC) % TWW, TWW};
+    const int m = n - NQ - NO;
+    if constexpr (!FULLHID) {
+        // step by step: the step's hidden tiles, then its two k-chunks of the second matmul
+        constexpr int SW_ = HT * KC + 2 * TWW;
+        const int st = m / SW_, r = m % SW_, base = BASE + st * SSTR;
+        if (r < HT * KC) return {base + KC * (r / KC) + r % KC, KC * HT};
+        return {base + 4 * KC + ((r - HT * KC) / TWW) * TW + (r - HT * KC) % TWW, TWW};
+    } else {
+        // every step's hidden tiles first, then the second matmul tile by tile over all k-chunks
+        // (the stream keeps the step-by-step order; chunk cc lies in step cc / 2)
+        constexpr int STEPS = TW, KCF = 2 * STEPS, NF1 = STEPS * HT * KC;
+        if (m < NF1) return {BASE + (m / (HT * KC)) * SSTR + m % (HT * KC), KC * HT};
+        const int i = (m - NF1) / KCF, cc = (m - NF1) % KCF;
+        return {BASE + (cc / 2) * SSTR + 4 * KC + (cc % 2) * TW + i, TWW};
+    }
 }
 
-template <int DM, bool TAPS, bool TWIN, bool FP8, bool OCTO = false>
+// Every wave's block sequence of a layer stays inside the layer's BPW blocks and the waves of a
+// quarter together visit each block exactly once (so no prefetch address leaves the stream: the
+// sequence only ever continues into the following layer or the head blocks).
+template <int KC, int TW, int SUB, int BPW, bool FULLHID>
+constexpr bool block_at_covers_layer() {
+    bool seen[BPW] = {};
+    for (int sub = 0; sub < SUB; sub++)
+        for (int n = 0; n < BPW / SUB; n++) {
+            const BlockAt at = block_at<KC, TW, SUB, FULLHID>(n);
+            const int i = at.a + sub * at.b;
+            if (i < 0 || i >= BPW || seen[i]) return false;
+            seen[i] = true;
+        }
+    return true;
+}
+
+template <int DM, bool TAPS, bool TWIN, bool FP8, bool OCTO = false, bool PROF = false>
 __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TWIN_OCC : 1) void board_kernel(const KArgs a) {
     typedef Cfg<DM, TWIN, OCTO> C;
     typedef typename Acc<FP8>::type acc_t;
@@ -159,17 +229,28 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     // register sets of the prefetch: NSETS - 1 half-blocks in flight
     constexpr int NSETS = OCTO ? BF_OCTO_SETS : BF_TWIN_SETS;
     static_assert(TW % SUB == 0 && (2 * NB) % NSETS == 0, "tiles and register sets must split evenly");
+    constexpr bool FULLHID = C::FULLHID;      // the whole quantised hidden row stays in LDS
+    static_assert(block_at_covers_layer<KC, TW, SUB, BPW, FULLHID>(), "block_at must enumerate a layer's blocks exactly once");
+    static_assert(!FULLHID || (STEPS == 2 && STEPS == TW && KCF == 2 * STEPS), "the full-row form is laid out for the 256-wide network");
+    static_assert(SLOTS <= HB && NSETS - 1 <= 2 * HB + 2, "the first prefetches of a heads-only run stay inside the head blocks");
     constexpr int XS = NW * 64;               // floats of one exchange slot
     // Eight wavefronts on the 512-wide network: a wave has 256 registers and the quantised row alone
     // would take 64 of them, so the activation fragments are read from LDS at each MFMA instead.
-    constexpr bool ACTL = OCTO && DM == 512;
+    constexpr bool ACTL = (OCTO && DM == 512) || BF_FORCE_ACTL;
     // One wave per SIMD (!TWIN, 512 registers): a tile's product is issued before the previous
     // tile's epilogue, and Q, K and V together, so the matrix pipe works under the vector work of
     // the same wave.  Two waves per SIMD (256 registers each): one product at a time, issued after
     // the previous epilogue -- the second set of accumulators would spill, and the SIMD's other
     // wave fills the gap.  Measured at batch 4096 (TWIN): 1.72 ms without a spill, against
     // 1.90 ms with 20 spilled registers when issuing ahead.
+    // int8 with one k-chunk per matmul of the width: the QKV, out-projection and first
+    // feed-forward accumulators start at the bit pattern of 1.5 * 2^23 (see chunk_sum), held in
+    // 16 registers that every such product reads as its addend.
+    constexpr bool BIASED = !FP8 && KC == 1 && BF_BIASED_ACC;
     constexpr bool AHEAD = !TWIN;
+    // In the feed-forward block of the full-row form the register file has room for the second
+    // accumulator at two waves per SIMD as well (only one tile's sums over the chunks are alive).
+    constexpr bool AH_FFN = AHEAD || (FULLHID && BF_TWIN_AHEAD_FFN);
     constexpr int HALF = BLOCK / 2;   // four fragments: the unit of the register prefetch (TWIN)
     constexpr int VM_AHEAD = TAPS ? 0 : (SLOTS - 1) * 8;   // ring loads that may stay in flight at a ring wait
     const int lane = threadIdx.x & 63;
@@ -181,12 +262,42 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     const int b = blockIdx.x;
     if (a.active && !a.active[b]) return;   // a skipped position: the whole workgroup leaves before any barrier
     const int nl_run = a.l1 - a.l0;
+    // Phase accounting (PROF builds only): the shader clock is read at phase boundaries and the
+    // cycles since the previous mark are charged to a slot; the time spent inside workgroup
+    // barriers is summed separately (and is also contained in the enclosing phases).
+    unsigned long long ph[N_PHASES];
+    unsigned long long t_mark = 0, t_begin = 0, t_sync = 0;
+    if constexpr (PROF) {
+#pragma unroll
+        for (int i = 0; i < N_PHASES; i++) ph[i] = 0;
+        t_mark = t_begin = __builtin_readcyclecounter();
+    }
+#define BF_PHASE(slot)                                                    \
+    do {                                                                  \
+        if constexpr (PROF) {                                             \
+            __builtin_amdgcn_sched_barrier(0); /* nothing is scheduled across the mark */ \
+            const unsigned long long now_ = __builtin_readcyclecounter(); \
+            __builtin_amdgcn_sched_barrier(0);                            \
+            ph[slot] += now_ - t_mark;                                    \
+            t_mark = now_;                                                \
+        }                                                                 \
+    } while (0)
+    auto barrier = [&]() {
+        if constexpr (PROF) {
+            const unsigned long long t0_ = __builtin_readcyclecounter();
+            lds_barrier();
+            t_sync += __builtin_readcyclecounter() - t0_;
+        } else {
+            lds_barrier();
+        }
+    };
 
     uint8_t* const myring = lds + wave * (SLOTS * BLOCK);   // !TWIN
     float* const xch = reinterpret_cast<float*>(lds + C::XCH_OFF);
     uint8_t* const hid = lds + C::HID_OFF;
     uint8_t* const act = lds + C::ACT_OFF;
-    float* const pA = reinterpret_cast<float*>(lds + C::PAR_OFF) + wave * C::PW_FLOATS;   // every wave keeps its own copy
+    float* const pA = reinterpret_cast<float*>(lds + C::PAR_OFF) + wave * C::PWL_FLOATS;   // every wave keeps its own copy
+    constexpr int B_COPY = C::BTAIL_GLOBAL ? C::B_LDS_FLOATS : C::B_FLOATS;
     float* const pB = pA + C::A_FLOATS;
     // the quarter's weight stream, from the first layer that runs; block `seq` in the quarter's order
     const uint8_t* const wsrc =
@@ -197,15 +308,25 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     // TWIN: half-block `hseq` of this wave's stream (consumption order) into register set `set`
     v4i frt[NSETS][4];
     auto load_half = [&](int hseq, int set) {
+#ifdef BF_EXP_SAMEBLOCK   // timing experiment: every weight load hits the same 4 KiB (L1 hits)
+        const uint8_t* src = wsrc + (size_t)(hseq & 1) * HALF;
+#else
         const uint8_t* src = wsrc + (size_t)hseq * HALF;
+#endif
+#ifdef BF_EXP_NOLOAD   // timing experiment: no weight traffic
+        (void)src;
+#pragma unroll
+        for (int s = 0; s < 4; s++) asm volatile("" : "=v"(frt[set][s]));
+#else
 #pragma unroll
         for (int s = 0; s < 4; s++) frt[set][s] = *reinterpret_cast<const v4i*>(src + s * FRAG);
+#endif
     };
     // the wave's hh-th half-block of the layer whose stream starts at block `base` (hh may run into
     // the following layer, whose stream starts at block `next`) into its register set
     auto fetch_half = [&](int hh, int base, int next) {
         const int n = hh / 2;
-        const BlockAt at = block_at<KC, TW, SUB>(n % NB);
+        const BlockAt at = block_at<KC, TW, SUB, FULLHID>(n % NB);
         load_half(2 * ((n < NB ? base : next) + at.a + sub * at.b) + hh % 2, hh % NSETS);
     };
     // !TWIN: block `seq` into ring slot `slot`; a slot into the fragment registers
@@ -231,14 +352,14 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     auto xsum = [&](auto&& chain, int slot) -> float {
         if constexpr (!OCTO) {
             xch[slot * XS + wave * 64 + lane] = chain(0.0f);
-            lds_barrier();
+            barrier();
             const float* p = xch + slot * XS + lane;
             return ((p[0] + p[64]) + p[128]) + p[192];
         } else {
             if (sub == 0) xch[q * 64 + lane] = chain(0.0f);
-            lds_barrier();
+            barrier();
             if (sub == 1) xch[XS + q * 64 + lane] = chain(xch[q * 64 + lane]);
-            lds_barrier();
+            barrier();
             const float* p = xch + XS + lane;
             return ((p[0] + p[64]) + p[128]) + p[192];
         }
@@ -287,7 +408,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
             for (int r = 0; r < 16; r++) am = __builtin_fmaxf(am, __builtin_fabsf(y[i][r]));
         xch[2 * XS + wave * 64 + lane] = am;
-        lds_barrier();
+        barrier();
 #pragma unroll
         for (int c = 0; c < KC; c++) {
             float m = 0.0f;   // the maximum is exact in any order: every wave of the chunk's quarters
@@ -312,7 +433,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 for (int j = 0; j < 4; j++)
                     *reinterpret_cast<int*>(tap + (tap_row * T + t) * D + 32 * (TW * q + t0 + i) + 8 * j + 4 * g) = w[j];
         }
-        lds_barrier();
+        barrier();
         if constexpr (!ACTL)
 #pragma unroll
             for (int n = 0; n < NT; n++) qv[n] = *reinterpret_cast<const v4i*>(act + n * FRAG + lane * 16);
@@ -327,17 +448,29 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         else return f.reg[s];
     };
 
+    acc_t acc_start = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (BIASED)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {   // opaque to the compiler, so the vector stays in registers
+            int m;
+            asm volatile("v_mov_b32 %0, 0x4b400000" : "=v"(m));
+            acc_start[r] = m;
+        }
+
     // ---- start the weight stream and the first layer's parameters ------------------------------
     if constexpr (TWIN) {
+        // a run of no layers (heads only) starts at the head blocks, which block_at does not
+        // describe: the stream is started below, where the heads restart it
+        if (nl_run > 0)
 #pragma unroll
-        for (int j = 0; j < NSETS - 1; j++) fetch_half(j, 0, BPW);
+            for (int j = 0; j < NSETS - 1; j++) fetch_half(j, 0, BPW);
     } else {
 #pragma unroll
-        for (int j = 0; j < SLOTS; j++) issue_block(j, j);
+        for (int j = 0; j < SLOTS; j++) issue_block(j, j);   // layer blocks, or the first head blocks (SLOTS <= HB)
     }
     if (nl_run > 0) {
         dma(wpar + (size_t)a.l0 * C::PW_FLOATS, pA, C::A_FLOATS, lane);
-        dma(wpar + (size_t)a.l0 * C::PW_FLOATS + C::A_FLOATS, pB, C::B_FLOATS, lane);
+        dma(wpar + (size_t)a.l0 * C::PW_FLOATS + C::A_FLOATS, pB, B_COPY, lane);
     }
 
     // ---- embedding (this wave's channels) --------------------------------------------------------
@@ -394,11 +527,14 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 
     wait_vm<0>();   // the parameters (and the first ring slots) have landed
     if constexpr (!TWIN) read_slot(0);
+    BF_PHASE(PH_EMBED);
 
     for (int l = a.l0; l < a.l1; l++) {
         const int li = l - a.l0;
         const size_t bl = (size_t)b * nl_run + li;   // tap row
         const int lnext = l + 1 < a.l1 ? l + 1 : l;  // after the last layer the same slice is fetched again
+        // the rarely read tail of the feed-forward parameters: in LDS with the rest, or in global memory
+        const float* const pBt = C::BTAIL_GLOBAL ? wpar + (size_t)l * C::PW_FLOATS + C::A_FLOATS : pB;
         // Multiply by the wave's k-th block of this layer (its own count: see block_at).
         // TWIN: its two halves sit in register sets 2k % NSETS and (2k + 1) % NSETS; a set is refilled
         // with the wave's half-block NSETS positions on once it has been consumed.  Four waves: that
@@ -407,7 +543,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         // !TWIN: the block is in `fr`; the ring slot it came from is refilled SLOTS blocks ahead,
         // then block k+1 is read from its slot.
         const int lbase = li * BPW, lfollow = OCTO ? (lnext - a.l0) * BPW : (li + 1) * BPW;
-#define BF_WMM(SWAP, k, actp) BF_WMM_FROM(SWAP, k, actp, (acc_t{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}))
+#define BF_WMM(SWAP, k, actp) BF_WMM_FROM(SWAP, k, actp, acc_start)
 #define BF_WMM_FROM(SWAP, k, actp, init)                                                             \
     ([&]() -> acc_t {                                                                                \
         const FragSrc act_ = (actp);                                                                 \
@@ -421,7 +557,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 r_ = frag_mma<SWAP>(frt[(2 * (k) + 1) % NSETS][s_], fragment(act_, 4 + s_), r_);     \
         } else {                                                                                     \
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                       \
-            issue_block(li * BPW + (k) + SLOTS, (k) % SLOTS);                                        \
+            issue_block(((k) + SLOTS < NB ? lbase : lfollow) + block_at<KC, TW, 1, FULLHID>(((k) + SLOTS) % NB).a, (k) % SLOTS); \
             _Pragma("unroll") for (int s_ = 0; s_ < 8; s_++)                                         \
                 r_ = frag_mma<SWAP>(fr[s_], fragment(act_, s_), r_);                                 \
             wait_vm<VM_AHEAD>();                                                                     \
@@ -438,6 +574,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             layernorm(x, pA + C::A_LN1G + 32 * t0, pA + C::A_LN1B + 32 * t0, y);
             quant_exchange(y, sa, xq, TAPS ? a.taps.qa_qkv : nullptr, bl);
         }
+        BF_PHASE(PH_LN1);
         float sa_tok[KC][16];   // activation scale of token ch(r, g), for the V tiles whose rows are tokens
         if constexpr (AHEAD)
 #pragma unroll
@@ -476,7 +613,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
-                    for (int k = 0; k < 4; k++) qf[4 * j + k] = chunk_sum<KC>(accq, 4 * j + k, sa) * swq + bq[j][k];
+                    for (int k = 0; k < 4; k++) qf[4 * j + k] = chunk_sum<KC, BIASED>(accq, 4 * j + k, sa) * swq + bq[j][k];
                 if constexpr (!AHEAD) {
                     pin16(qf);
 #pragma unroll
@@ -485,7 +622,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
                 for (int j = 0; j < 4; j++)
 #pragma unroll
-                    for (int k = 0; k < 4; k++) kf[4 * j + k] = chunk_sum<KC>(acck, 4 * j + k, sa) * swk + bk[j][k];
+                    for (int k = 0; k < 4; k++) kf[4 * j + k] = chunk_sum<KC, BIASED>(acck, 4 * j + k, sa) * swk + bk[j][k];
                 if constexpr (!AHEAD) {
                     pin16(kf);
 #pragma unroll
@@ -496,7 +633,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                     float st[KC];
 #pragma unroll
                     for (int c = 0; c < KC; c++) st[c] = AHEAD ? sa_tok[c][r] : __shfl(sa[c], ch(r, g));
-                    vf[r] = chunk_sum<KC>(accv, r, st) * swv + bv;
+                    vf[r] = chunk_sum<KC, BIASED>(accv, r, st) * swv + bv;
                 }
                 if (TAPS && a.taps.acc_qkv)
 #pragma unroll
@@ -504,15 +641,16 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
                             int* row = a.taps.acc_qkv + ((bl * KC + c) * T + t) * 3 * D;
-                            row[32 * h + ch(r, g)] = accbits(accq[c], r);
-                            row[D + 32 * h + ch(r, g)] = accbits(acck[c], r);
-                            a.taps.acc_qkv[((bl * KC + c) * T + ch(r, g)) * 3 * D + 2 * D + 32 * h + t] = accbits(accv[c], r);
+                            row[32 * h + ch(r, g)] = tapbits<BIASED>(accq[c], r);
+                            row[D + 32 * h + ch(r, g)] = tapbits<BIASED>(acck[c], r);
+                            a.taps.acc_qkv[((bl * KC + c) * T + ch(r, g)) * 3 * D + 2 * D + 32 * h + t] = tapbits<BIASED>(accv[c], r);
                         }
             }
+            BF_PHASE(PH_QKV);
             // scores, transposed: lane = query token, register r = key ch(r, g)
             v16f sc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int r = 0; r < 16; r++) sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[r], qf[r], sc, 0, 0, 0);
+            for (int r = 0; r < 16; r++) sc = BF_F32MMA(kf[r], qf[r], sc);
             if (AHEAD && i + 1 < TWW) {
 #pragma unroll
                 for (int c = 0; c < KC; c++) accq[c] = BF_WMM(false, 3 * KC * (i + 1) + c, fragments(xq, act, 8 * c));
@@ -540,9 +678,10 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             const float rl = 1.0f / (lsum + partner(lsum, g));
             v16f oa = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int r = 0; r < 16; r++) oa = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[r], p[r] * rl, oa, 0, 0, 0);
+            for (int r = 0; r < 16; r++) oa = BF_F32MMA(vf[r], p[r] * rl, oa);
 #pragma unroll
             for (int r = 0; r < 16; r++) o[i][r] = oa[r];
+            BF_PHASE(PH_ATTN);
         }
 
         // ---- output projection + residual (this wave's output tiles) -----------------------------------
@@ -566,19 +705,20 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 for (int j = 0; j < 4; j++)
 #pragma unroll
                     for (int k = 0; k < 4; k++)
-                        x[i][4 * j + k] = x[i][4 * j + k] + (chunk_sum<KC>(acc2[AHEAD ? i & 1 : 0], 4 * j + k, so) * sw + bo[j][k]);
+                        x[i][4 * j + k] = x[i][4 * j + k] + (chunk_sum<KC, BIASED>(acc2[AHEAD ? i & 1 : 0], 4 * j + k, so) * sw + bo[j][k]);
                 pin16(x[i]);
                 if (TAPS && a.taps.acc_out)
 #pragma unroll
                     for (int c = 0; c < KC; c++)
 #pragma unroll
                         for (int r = 0; r < 16; r++)
-                            a.taps.acc_out[((bl * KC + c) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = accbits(acc2[AHEAD ? i & 1 : 0][c], r);
+                            a.taps.acc_out[((bl * KC + c) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = tapbits<BIASED>(acc2[AHEAD ? i & 1 : 0][c], r);
                 if (!AHEAD && i + 1 < TWW)
 #pragma unroll
                     for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, K0 + KC * (i + 1) + c, fragments(oq, act, 8 * c));
             }
         }
+        BF_PHASE(PH_OUT);
         // the attention-phase parameters are dead: fetch the next layer's
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         dma(wpar + (size_t)lnext * C::PW_FLOATS, pA, C::A_FLOATS, lane);
@@ -589,15 +729,17 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             layernorm(x, pB + C::B_LN2G + 32 * t0, pB + C::B_LN2B + 32 * t0, y);
             quant_exchange(y, sa, xq, TAPS ? a.taps.qa_ff1 : nullptr, bl);
         }
-        double o64[TWW][16];   // int8: float64 sums over the k-chunks
-        float o32[TWW][16];    // e4m3: fp32 sums over the k-tiles
+        BF_PHASE(PH_LN2);
         constexpr int KF = 3 * KC * TWW + KC * TWW;   // the wave's first feed-forward block of the layer
+        if constexpr (FULLHID) {
+            // First matmul of every step, each step's two 256-wide chunks quantised as soon as the
+            // step is complete (a chunk spans a pair of quarters: waves 0,1 the step's first chunk,
+            // 2,3 its second); the whole quantised hidden row stays in LDS.  int8: unsigned, bytes
+            // stored as q - 128 for the signed MFMA; e4m3: the ordinary signed quantiser.
+            float sh[KCF];
 #pragma unroll
-        for (int st = 0; st < STEPS; st++) {
-            constexpr int SBLK = HT * KC + 2 * TWW;   // the wave's blocks of one step
-            const int k1 = KF + st * SBLK;            // first matmul: HT hidden tiles of this wave (of the 16 of a step)
-            float sh[2];                              // scales of the step's two chunks
-            {
+            for (int st = 0; st < STEPS; st++) {
+                const int k1 = KF + st * HT * KC;
                 float hf[HT][16];
                 float am = 0.0f;
                 acc_t acc2[2][KC];
@@ -605,17 +747,20 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + c, fragments(xq, act, 8 * c));
 #pragma unroll
                 for (int i = 0; i < HT; i++) {
-                    if (AHEAD && i + 1 < HT)
+                    if (AH_FFN && i + 1 < HT)
 #pragma unroll
                         for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, k1 + KC * (i + 1) + c, fragments(xq, act, 8 * c));
                     v4f b1[4];
-                    load_tile16(pB + C::B_BFF1 + 128 * st + 32 * (h0 + i), g, b1);
+                    load_tile16(pBt + C::B_BFF1 + 128 * st + 32 * (h0 + i), g, b1);
                     const float sw = pB[C::B_SW + 4 * st + h0 + i];
 #pragma unroll
                     for (int j = 0; j < 4; j++)
 #pragma unroll
                         for (int k = 0; k < 4; k++) {
-                            const float v = __builtin_fmaxf(chunk_sum<KC>(acc2[AHEAD ? i & 1 : 0], 4 * j + k, sa) * sw + b1[j][k], 0.0f);
+                            // int8: the ReLU is the saturation of the unsigned quantiser below, and the
+                            // running maximum starts at 0, so negative values need no clamp here
+                            float v = chunk_sum<KC, BIASED>(acc2[AH_FFN ? i & 1 : 0], 4 * j + k, sa) * sw + b1[j][k];
+                            if constexpr (FP8) v = __builtin_fmaxf(v, 0.0f);
                             hf[i][4 * j + k] = v;
                             am = __builtin_fmaxf(am, v);
                         }
@@ -625,58 +770,55 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                         for (int c = 0; c < KC; c++)
 #pragma unroll
                             for (int r = 0; r < 16; r++)
-                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + ch(r, g)] = accbits(acc2[AHEAD ? i & 1 : 0][c], r);
-                    if (!AHEAD && i + 1 < HT)
+                                a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + ch(r, g)] = tapbits<BIASED>(acc2[AH_FFN ? i & 1 : 0][c], r);
+                    if (!AH_FFN && i + 1 < HT)
 #pragma unroll
                         for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + KC * (i + 1) + c, fragments(xq, act, 8 * c));
                 }
-                // quantiser over the 256-wide chunk this wave shares with its neighbour (waves 0,1: first
-                // chunk of the step; 2,3: second).  int8: unsigned, bytes stored as q - 128 for the signed
-                // MFMA; e4m3: the ordinary signed quantiser (the values are non-negative)
-                xch[2 * XS + wave * 64 + lane] = am;
-                lds_barrier();
+                // the maxima of consecutive steps go through different exchange slots (2, then 0, whose
+                // last use was the LayerNorm sum several barriers ago): a fast wave's next maximum
+                // must not overwrite what a slow wave still reads
+                const int xs = (st & 1) ? 0 : 2 * XS;
+                xch[xs + wave * 64 + lane] = am;
+                barrier();
 #pragma unroll
                 for (int c = 0; c < 2; c++) {
                     float m = 0.0f;   // hidden values are >= 0
 #pragma unroll
                     for (int u = 0; u < SUB; u++)
-                        m = __builtin_fmaxf(m, __builtin_fmaxf(xch[2 * XS + (2 * c + 4 * u) * 64 + lane],
-                                                               xch[2 * XS + (2 * c + 1 + 4 * u) * 64 + lane]));
+                        m = __builtin_fmaxf(m, __builtin_fmaxf(xch[xs + (2 * c + 4 * u) * 64 + lane],
+                                                               xch[xs + (2 * c + 1 + 4 * u) * 64 + lane]));
                     m = __builtin_fmaxf(m, partner(m, g));
-                    sh[c] = m > 0.0f ? m / (FP8 ? 8.0f : 255.0f) : 1.0f;
+                    sh[2 * st + c] = m > 0.0f ? m / (FP8 ? 8.0f : 255.0f) : 1.0f;
                 }
-                const float s8 = q < 2 ? sh[0] : sh[1];
+                const float s8 = q < 2 ? sh[2 * st] : sh[2 * st + 1];
                 const float inv = 1.0f / s8;
 #pragma unroll
                 for (int i = 0; i < HT; i++) {
                     v4i w;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        const unsigned u = quant4<FP8>(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
+                        unsigned u;
+                        if constexpr (FP8) u = quant4<true>(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
+                        else u = quant4_relu_u8(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
                         if (TAPS && a.taps.qa_ff2)
                             *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + 8 * j + 4 * g) = u;
                         w[j] = (int)(FP8 ? u : (u ^ 0x80808080u));
                     }
-                    *reinterpret_cast<v4i*>(hid + (4 * q + h0 + i) * FRAG + lane * 16) = w;
+                    *reinterpret_cast<v4i*>(hid + (16 * st + 4 * q + h0 + i) * FRAG + lane * 16) = w;
                 }
             }
-            lds_barrier();
-            // second matmul, chunk-major: one chunk of the hidden row (eight fragments) serves this
-            // wave's TW output tiles; the float64 sums over the chunks stay in chunk order
-            const int k2 = k1 + HT * KC;
-            acc_t acc2[2];
-            v4i hqc[8];
-            if constexpr (!ACTL)
-#pragma unroll
-                for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + s * FRAG + lane * 16);
-            // int8, one product at a time: the accumulator starts at 128 * sum(w) (the offset of the
-            // unsigned operand bytes stored as q - 128), which saves adding it afterwards
-            constexpr bool WFOLD = !AHEAD && !FP8;
+            barrier();   // the whole hidden row is in LDS
+            BF_PHASE(PH_FF1);
+            // Second matmul, tile by tile: the KCF k-chunks of one output tile in turn, so only one
+            // tile's sums over the chunks (float64 for int8, fp32 for e4m3) are alive.  int8: the
+            // accumulator starts at 128 * sum(w), the offset of the unsigned bytes stored as q - 128.
+            constexpr int K2 = KF + STEPS * HT * KC, N2 = TWW * KCF;
             auto wsum_start = [&](int idx) -> acc_t {
                 acc_t r = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                if constexpr (WFOLD) {
+                if constexpr (!FP8) {
                     v4i w0[4];
-                    load_tile16i(pB + C::B_WSUM + (2 * st + idx / TWW) * CW + 32 * (t0 + idx % TWW), g, w0);
+                    load_tile16i(pBt + C::B_WSUM + (idx % KCF) * CW + 32 * (t0 + idx / KCF), g, w0);
 #pragma unroll
                     for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -684,72 +826,234 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 }
                 return r;
             };
-            acc2[0] = BF_WMM_FROM(false, k2, fragments(hqc, hid, 0), wsum_start(0));
+            auto product = [&](int idx) -> acc_t {
+                const int cc = idx % KCF;
+                v4i hqc[8];
+                if constexpr (!ACTL)
 #pragma unroll
-            for (int idx = 0; idx < 2 * TWW; idx++) {
-                const int c = idx / TWW, i = idx % TWW;
-                v4i ws[4] = {};
-                if (!FP8 && !WFOLD) load_tile16i(pB + C::B_WSUM + (2 * st + c) * CW + 32 * (t0 + i), g, ws);
-                if (AHEAD && idx + 1 < 2 * TWW) {
-                    if ((idx + 1) % TWW == 0)
+                    for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * cc + s) * FRAG + lane * 16);
+                return BF_WMM_FROM(false, K2 + idx, (FragSrc{&hqc[0], hid + 8 * cc * FRAG + lane * 16}), wsum_start(idx));
+            };
+            acc_t accp[2];
+            accp[0] = product(0);
+            double o64[16];
+            float o32[16];
 #pragma unroll
-                        for (int s = 0; s < 8; s++)
-                            hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * (c + 1) + s) * FRAG + lane * 16);
-                    acc2[(idx + 1) & 1] = BF_WMM(false, k2 + idx + 1, fragments(hqc, hid, 0));
-                }
-                if (!AHEAD && idx > 0) {
-                    if (!ACTL && idx % TWW == 0)   // the next chunk of the hidden row
-#pragma unroll
-                        for (int s = 0; s < 8; s++)
-                            hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * c + s) * FRAG + lane * 16);
-                    acc2[0] = BF_WMM_FROM(false, k2 + idx, (FragSrc{&hqc[0], hid + 8 * c * FRAG + lane * 16}), wsum_start(idx));
-                }
-                const acc_t acc = acc2[AHEAD ? idx & 1 : 0];
+            for (int idx = 0; idx < N2; idx++) {
+                const int i = idx / KCF, cc = idx % KCF;
+                if (AH_FFN && idx + 1 < N2) accp[(idx + 1) & 1] = product(idx + 1);
+                const acc_t acc = accp[AH_FFN ? idx & 1 : 0];
                 if constexpr (FP8) {
                     // descale each 256-deep tile with its own scales, fp32 sum over the tiles
-                    const float sw = pB[C::B_SW + 16 + (t0 + i) * KCF + 2 * st + c];
+                    const float sw = pB[C::B_SW + 16 + (t0 + i) * KCF + cc];
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        const float part = (accf(acc, r) * sh[c]) * sw;
-                        o32[i][r] = (st == 0 && c == 0) ? part : o32[i][r] + part;
+                        const float part = (accf(acc, r) * sh[cc]) * sw;
+                        o32[r] = cc == 0 ? part : o32[r] + part;
                         if (TAPS && a.taps.acc_ff2)
-                            a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = accbits(acc, r);
+                            a.taps.acc_ff2[((bl * KCF + cc) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = accbits(acc, r);
                     }
-                    pin16(o32[i]);
+                    pin16(o32);
                 } else {
-                    const double sc = (double)sh[c];
+                    const double sc = (double)sh[cc];
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int full = accbits(acc, r);
+                        o64[r] = cc == 0 ? (double)full * sc : __builtin_fma((double)full, sc, o64[r]);
+                        if (TAPS && a.taps.acc_ff2)
+                            a.taps.acc_ff2[((bl * KCF + cc) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = full;
+                    }
+#pragma unroll
+                    for (int r = 0; r < 16; r++) pin(o64[r]);
+                }
+                if (cc == KCF - 1) {
+                    v4f b2[4];
+                    load_tile16(pB + C::B_BFF2 + 32 * (t0 + i), g, b2);
+                    const float sw = pB[C::B_SW + 16 + t0 + i];
 #pragma unroll
                     for (int j = 0; j < 4; j++)
 #pragma unroll
                         for (int k = 0; k < 4; k++) {
-                            const int full = WFOLD ? accbits(acc, 4 * j + k) : accbits(acc, 4 * j + k) + ws[j][k];
-                            o64[i][4 * j + k] = (st == 0 && c == 0) ? (double)full * sc
-                                                                    : __builtin_fma((double)full, sc, o64[i][4 * j + k]);
-                            if (TAPS && a.taps.acc_ff2)
-                                a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * q + t0 + i) + 8 * j + 4 * g + k] = full;
+                            float upd;
+                            if constexpr (FP8) upd = o32[4 * j + k] + b2[j][k];
+                            else upd = (float)o64[4 * j + k] * sw + b2[j][k];
+                            x[i][4 * j + k] = x[i][4 * j + k] + upd;
                         }
-#pragma unroll
-                    for (int r = 0; r < 16; r++) pin(o64[i][r]);
+                    pin16(x[i]);
                 }
+                if (!AH_FFN && idx + 1 < N2) accp[0] = product(idx + 1);
+            }
+            BF_PHASE(PH_FF2);
+        } else {
+            double o64[TWW][16];   // int8: float64 sums over the k-chunks
+            float o32[TWW][16];    // e4m3: fp32 sums over the k-tiles
+#pragma unroll
+            for (int st = 0; st < STEPS; st++) {
+                constexpr int SBLK = HT * KC + 2 * TWW;   // the wave's blocks of one step
+                const int k1 = KF + st * SBLK;            // first matmul: HT hidden tiles of this wave (of the 16 of a step)
+                float sh[2];                              // scales of the step's two chunks
+                {
+                    float hf[HT][16];
+                    float am = 0.0f;
+                    acc_t acc2[2][KC];
+#pragma unroll
+                    for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + c, fragments(xq, act, 8 * c));
+#pragma unroll
+                    for (int i = 0; i < HT; i++) {
+                        if (AHEAD && i + 1 < HT)
+#pragma unroll
+                            for (int c = 0; c < KC; c++) acc2[(i + 1) & 1][c] = BF_WMM(false, k1 + KC * (i + 1) + c, fragments(xq, act, 8 * c));
+                        v4f b1[4];
+                        load_tile16(pBt + C::B_BFF1 + 128 * st + 32 * (h0 + i), g, b1);
+                        const float sw = pB[C::B_SW + 4 * st + h0 + i];
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+#pragma unroll
+                            for (int k = 0; k < 4; k++) {
+                                // int8: the ReLU is the saturation of the unsigned quantiser below, and the
+                                // running maximum starts at 0, so negative values need no clamp here
+                                float v = chunk_sum<KC, BIASED>(acc2[AHEAD ? i & 1 : 0], 4 * j + k, sa) * sw + b1[j][k];
+                                if constexpr (FP8) v = __builtin_fmaxf(v, 0.0f);
+                                hf[i][4 * j + k] = v;
+                                am = __builtin_fmaxf(am, v);
+                            }
+                        pin16(hf[i]);
+                        if (TAPS && a.taps.acc_ff1)
+#pragma unroll
+                            for (int c = 0; c < KC; c++)
+#pragma unroll
+                                for (int r = 0; r < 16; r++)
+                                    a.taps.acc_ff1[((bl * KC + c) * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + ch(r, g)] = tapbits<BIASED>(acc2[AHEAD ? i & 1 : 0][c], r);
+                        if (!AHEAD && i + 1 < HT)
+#pragma unroll
+                            for (int c = 0; c < KC; c++) acc2[0][c] = BF_WMM(false, k1 + KC * (i + 1) + c, fragments(xq, act, 8 * c));
+                    }
+                    // quantiser over the 256-wide chunk this wave shares with its neighbour (waves 0,1: first
+                    // chunk of the step; 2,3: second).  int8: unsigned, bytes stored as q - 128 for the signed
+                    // MFMA; e4m3: the ordinary signed quantiser (the values are non-negative)
+                    xch[2 * XS + wave * 64 + lane] = am;
+                    barrier();
+#pragma unroll
+                    for (int c = 0; c < 2; c++) {
+                        float m = 0.0f;   // hidden values are >= 0
+#pragma unroll
+                        for (int u = 0; u < SUB; u++)
+                            m = __builtin_fmaxf(m, __builtin_fmaxf(xch[2 * XS + (2 * c + 4 * u) * 64 + lane],
+                                                                   xch[2 * XS + (2 * c + 1 + 4 * u) * 64 + lane]));
+                        m = __builtin_fmaxf(m, partner(m, g));
+                        sh[c] = m > 0.0f ? m / (FP8 ? 8.0f : 255.0f) : 1.0f;
+                    }
+                    const float s8 = q < 2 ? sh[0] : sh[1];
+                    const float inv = 1.0f / s8;
+#pragma unroll
+                    for (int i = 0; i < HT; i++) {
+                        v4i w;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            unsigned u;
+                            if constexpr (FP8) u = quant4<true>(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
+                            else u = quant4_relu_u8(hf[i][4 * j], hf[i][4 * j + 1], hf[i][4 * j + 2], hf[i][4 * j + 3], s8, inv);
+                            if (TAPS && a.taps.qa_ff2)
+                                *reinterpret_cast<unsigned*>(a.taps.qa_ff2 + (bl * T + t) * F + 512 * st + 128 * q + 32 * (h0 + i) + 8 * j + 4 * g) = u;
+                            w[j] = (int)(FP8 ? u : (u ^ 0x80808080u));
+                        }
+                        *reinterpret_cast<v4i*>(hid + (4 * q + h0 + i) * FRAG + lane * 16) = w;
+                    }
+                }
+                barrier();
+                BF_PHASE(PH_FF1);
+                // second matmul, chunk-major: one chunk of the hidden row (eight fragments) serves this
+                // wave's TW output tiles; the float64 sums over the chunks stay in chunk order
+                const int k2 = k1 + HT * KC;
+                acc_t acc2[2];
+                v4i hqc[8];
+                if constexpr (!ACTL)
+#pragma unroll
+                    for (int s = 0; s < 8; s++) hqc[s] = *reinterpret_cast<const v4i*>(hid + s * FRAG + lane * 16);
+                // int8, one product at a time: the accumulator starts at 128 * sum(w) (the offset of the
+                // unsigned operand bytes stored as q - 128), which saves adding it afterwards
+                constexpr bool WFOLD = !AHEAD && !FP8;
+                auto wsum_start = [&](int idx) -> acc_t {
+                    acc_t r = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    if constexpr (WFOLD) {
+                        v4i w0[4];
+                        load_tile16i(pBt + C::B_WSUM + (2 * st + idx / TWW) * CW + 32 * (t0 + idx % TWW), g, w0);
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+#pragma unroll
+                            for (int k = 0; k < 4; k++) r[4 * j + k] = w0[j][k];
+                    }
+                    return r;
+                };
+                acc2[0] = BF_WMM_FROM(false, k2, fragments(hqc, hid, 0), wsum_start(0));
+#pragma unroll
+                for (int idx = 0; idx < 2 * TWW; idx++) {
+                    const int c = idx / TWW, i = idx % TWW;
+                    v4i ws[4] = {};
+                    if (!FP8 && !WFOLD) load_tile16i(pBt + C::B_WSUM + (2 * st + c) * CW + 32 * (t0 + i), g, ws);
+                    if (AHEAD && idx + 1 < 2 * TWW) {
+                        if ((idx + 1) % TWW == 0)
+#pragma unroll
+                            for (int s = 0; s < 8; s++)
+                                hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * (c + 1) + s) * FRAG + lane * 16);
+                        acc2[(idx + 1) & 1] = BF_WMM(false, k2 + idx + 1, fragments(hqc, hid, 0));
+                    }
+                    if (!AHEAD && idx > 0) {
+                        if (!ACTL && idx % TWW == 0)   // the next chunk of the hidden row
+#pragma unroll
+                            for (int s = 0; s < 8; s++)
+                                hqc[s] = *reinterpret_cast<const v4i*>(hid + (8 * c + s) * FRAG + lane * 16);
+                        acc2[0] = BF_WMM_FROM(false, k2 + idx, (FragSrc{&hqc[0], hid + 8 * c * FRAG + lane * 16}), wsum_start(idx));
+                    }
+                    const acc_t acc = acc2[AHEAD ? idx & 1 : 0];
+                    if constexpr (FP8) {
+                        // descale each 256-deep tile with its own scales, fp32 sum over the tiles
+                        const float sw = pB[C::B_SW + 16 + (t0 + i) * KCF + 2 * st + c];
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const float part = (accf(acc, r) * sh[c]) * sw;
+                            o32[i][r] = (st == 0 && c == 0) ? part : o32[i][r] + part;
+                            if (TAPS && a.taps.acc_ff2)
+                                a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = accbits(acc, r);
+                        }
+                        pin16(o32[i]);
+                    } else {
+                        const double sc = (double)sh[c];
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+#pragma unroll
+                            for (int k = 0; k < 4; k++) {
+                                const int full = WFOLD ? accbits(acc, 4 * j + k) : accbits(acc, 4 * j + k) + ws[j][k];
+                                o64[i][4 * j + k] = (st == 0 && c == 0) ? (double)full * sc
+                                                                        : __builtin_fma((double)full, sc, o64[i][4 * j + k]);
+                                if (TAPS && a.taps.acc_ff2)
+                                    a.taps.acc_ff2[((bl * KCF + 2 * st + c) * T + t) * D + 32 * (TW * q + t0 + i) + 8 * j + 4 * g + k] = full;
+                            }
+#pragma unroll
+                        for (int r = 0; r < 16; r++) pin(o64[i][r]);
+                    }
+                }
+                BF_PHASE(PH_FF2);
+            }
+#pragma unroll
+            for (int i = 0; i < TWW; i++) {
+                v4f b2[4];
+                load_tile16(pB + C::B_BFF2 + 32 * (t0 + i), g, b2);
+                const float sw = pB[C::B_SW + 16 + t0 + i];
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        float upd;
+                        if constexpr (FP8) upd = o32[i][4 * j + k] + b2[j][k];
+                        else upd = (float)o64[i][4 * j + k] * sw + b2[j][k];
+                        x[i][4 * j + k] = x[i][4 * j + k] + upd;
+                    }
             }
         }
-#pragma unroll
-        for (int i = 0; i < TWW; i++) {
-            v4f b2[4];
-            load_tile16(pB + C::B_BFF2 + 32 * (t0 + i), g, b2);
-            const float sw = pB[C::B_SW + 16 + t0 + i];
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    float upd;
-                    if constexpr (FP8) upd = o32[i][4 * j + k] + b2[j][k];
-                    else upd = (float)o64[i][4 * j + k] * sw + b2[j][k];
-                    x[i][4 * j + k] = x[i][4 * j + k] + upd;
-                }
-        }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        dma(wpar + (size_t)lnext * C::PW_FLOATS + C::A_FLOATS, pB, C::B_FLOATS, lane);
+        dma(wpar + (size_t)lnext * C::PW_FLOATS + C::A_FLOATS, pB, B_COPY, lane);
+        BF_PHASE(PH_FF2);
 #undef BF_WMM
 #undef BF_WMM_FROM
         if (TAPS && a.taps.resid)
@@ -765,7 +1069,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     // the blocks of the next layer there: then restart the stream at the head blocks.
     const int hseq0 = (a.n_layers - a.l0) * BPW;
     wait_vm<0>();   // also: no parameter copy is still landing where the normalised stream goes
-    if (OCTO || a.l1 != a.n_layers) {
+    if (OCTO || a.l1 != a.n_layers || (TWIN && nl_run == 0)) {
         if constexpr (TWIN) {
 #pragma unroll
             for (int j = 0; j < NSETS - 1; j++) load_half(2 * hseq0 + j, j);
@@ -794,7 +1098,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             const v4f v = {hn[i][4 * j], hn[i][4 * j + 1], hn[i][4 * j + 2], hn[i][4 * j + 3]};
             *reinterpret_cast<v4f*>(hnb + (((TW * q + t0 + i) * 4 + j) * 64 + lane) * 4) = v;
         }
-    lds_barrier();
+    barrier();
     // The first wave of quarter m multiplies head tile m (rows 32m..32m+31 of [policy; promo;
     // value; 0]) over the whole width, one fused-multiply-add chain in (tile, quad, element) order;
     // quarter 3's tile is zero.  With eight waves the second wave of a quarter has nothing to
@@ -834,6 +1138,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         }
     }
 
+    BF_PHASE(PH_HEADS);
     // value: king token of the side to move, lane half 1 of head tile 2 holds rows 68..70
     if (heads_here && q == 2) {
         const int king = ctrl < 0 ? 31 : 15;
@@ -900,7 +1205,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             xch[q * 2] = bv;
             xch[q * 2 + 1] = __int_as_float(bi);
         }
-        lds_barrier();
+        barrier();
         if (wave == 0 && lane == 0) {
             const float ov = xch[2];
             const int oi = __float_as_int(xch[3]);
@@ -909,20 +1214,33 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             a.best[b] = bi == 0x7fffffff ? -1 : bi;
         }
     }
+    if constexpr (PROF) {
+        BF_PHASE(PH_STORE);
+        ph[PH_SYNC] = t_sync;
+        ph[PH_TOTAL] = __builtin_readcyclecounter() - t_begin;
+        if (lane == 0 && a.profile)
+#pragma unroll
+            for (int i = 0; i < N_PHASES; i++) atomicAdd(&a.profile[i], ph[i]);
+    }
+#undef BF_PHASE
 }
 
-template <int DM, bool TAPS, bool TWIN, bool FP8 = false, bool OCTO = false>
+template <int DM, bool TAPS, bool TWIN, bool FP8 = false, bool OCTO = false, bool PROF = false>
 hipError_t launch_board(const KArgs& k, hipStream_t stream) {
-    // more than 64 KiB of dynamic LDS has to be requested once per kernel (per thread: cheap)
-    static thread_local bool lds_set = false;
+    // more than 64 KiB of dynamic LDS has to be requested once per kernel and device (one bit
+    // per device ordinal; a device beyond the mask asks every time)
+    static std::atomic<unsigned long long> lds_set{0};
     constexpr int lds_bytes = Cfg<DM, TWIN, OCTO>::LDS_BYTES;
-    if (!lds_set) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&board_kernel<DM, TAPS, TWIN, FP8, OCTO>),
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return hipErrorInvalidDevice;
+    const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
+    if (!(lds_set.load(std::memory_order_relaxed) & bit)) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&board_kernel<DM, TAPS, TWIN, FP8, OCTO, PROF>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess) return e;
-        lds_set = true;
+        lds_set.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((board_kernel<DM, TAPS, TWIN, FP8, OCTO>), dim3(k.n), dim3(OCTO ? 2 * THREADS : THREADS), lds_bytes, stream, k);
+    hipLaunchKernelGGL((board_kernel<DM, TAPS, TWIN, FP8, OCTO, PROF>), dim3(k.n), dim3(OCTO ? 2 * THREADS : THREADS), lds_bytes, stream, k);
     return hipGetLastError();
 }
 

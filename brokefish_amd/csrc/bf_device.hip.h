@@ -171,6 +171,23 @@ __device__ __forceinline__ unsigned quant4(float v0, float v1, float v2, float v
     }
 }
 
+// The unsigned int8 quantiser of the feed-forward hidden row with the ReLU folded in: four
+// correctly rounded quotients v / sa, converted with v_cvt_pk_u8_f32 -- round to nearest even,
+// saturating to [0, 255], so a negative input gives 0 exactly as max(v, 0) would (checked on the
+// GPU against rint + clamp on two million values and every tie k + 0.5) -- each conversion
+// writing its own byte of the dword.
+__device__ __forceinline__ unsigned quant4_relu_u8(float v0, float v1, float v2, float v3, float sa, float inv) {
+    const float v[4] = {v0, v1, v2, v3};
+    unsigned w = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float q0 = v[i] * inv;
+        const float rem = __builtin_fmaf(-q0, sa, v[i]);
+        w = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(rem, inv, q0), i, w);
+    }
+    return w;
+}
+
 // signed quantiser (int8: amax -> 127, e4m3: amax -> 8) of one token row spread over two
 // lanes; y is [tiles][16]
 template <int NTILES, bool FP8>

@@ -2,6 +2,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 
@@ -173,25 +174,51 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     return BF_OK;
 }
 
+// Whether the current device is an MI355X-class part (gfx950), looked up once per device; the
+// kernels are compiled for that architecture only.
+static bool device_is_gfx950() {
+    static std::atomic<unsigned long long> known{0}, good{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        fail(BF_ERR_DEVICE, "no current HIP device");
+        return false;
+    }
+    const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
+    bool ok;
+    if (known.load(std::memory_order_acquire) & bit) {
+        ok = good.load(std::memory_order_relaxed) & bit;
+    } else {
+        hipDeviceProp_t prop;
+        ok = hipGetDeviceProperties(&prop, dev) == hipSuccess && strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+        if (ok) good.fetch_or(bit, std::memory_order_relaxed);
+        known.fetch_or(bit, std::memory_order_release);
+    }
+    if (!ok) fail(BF_ERR_DEVICE, "the current device is not a gfx950 GPU: the kernels of this library are built for MI355X only");
+    return ok;
+}
+
 static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream_t stream) {
     const int grid = (k.n + bf::WAVES - 1) / bf::WAVES;
     hipError_t e;
+    if (!device_is_gfx950()) return BF_ERR_DEVICE;
     if (kind == BF_KERNEL_OCTO) {
-        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
-        if (a->shape.d_model == 512)
+        if (k.profile)
+            e = a->shape.d_model == 512 ? bf::launch_octo512_prof(k, stream) : bf::launch_octo256_prof(k, stream);
+        else if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_octo512_taps(k, stream) : bf::launch_octo512(k, stream);
         else if (a->quant == BF_QUANT_E4M3)
             e = a->taps ? bf::launch_octo256_fp8_taps(k, stream) : bf::launch_octo256_fp8(k, stream);
         else
             e = a->taps ? bf::launch_octo256_taps(k, stream) : bf::launch_octo256(k, stream);
     } else if (kind == BF_KERNEL_TWIN) {
-        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
-        if (a->quant == BF_QUANT_E4M3)
+        if (k.profile)
+            e = bf::launch_twin256_prof(k, stream);
+        else if (a->quant == BF_QUANT_E4M3)
             e = a->taps ? bf::launch_twin256_fp8_taps(k, stream) : bf::launch_twin256_fp8(k, stream);
         else
             e = a->taps ? bf::launch_twin256_taps(k, stream) : bf::launch_twin256(k, stream);
     } else if (kind == BF_KERNEL_BOARD) {
-        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the four-positions-per-workgroup kernel");
+        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the TWIN, OCTO and QUAD kernels");
         if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_board512_taps(k, stream) : bf::launch_board512(k, stream);
         else if (a->quant == BF_QUANT_E4M3)
@@ -284,6 +311,7 @@ extern "C" int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_
     if (rc) return rc;
     if (args->taps) return fail(BF_ERR_ARGUMENT, "the phase profile runs without taps");
     if (args->quant != BF_QUANT_INT8) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the int8 format only");
+    if (kind == BF_KERNEL_BOARD) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the TWIN, OCTO and QUAD kernels");
     if (!cycles) return fail(BF_ERR_ARGUMENT, "cycles must not be NULL");
     k.profile = reinterpret_cast<unsigned long long*>(cycles);
     return launch(args, k, kind, (hipStream_t)stream);
@@ -294,7 +322,7 @@ extern "C" int bf_profile_phase_count(void) { return bf::N_PHASES; }
 extern "C" const char* bf_profile_phase_name(int i) {
     static const char* names[bf::N_PHASES] = {"embed", "ln1_quant", "qkv_gemm_epilogue", "attention",
                                               "oquant_outproj", "ln2_quant", "ffn1", "ffn2", "heads",
-                                              "store", "ring_wait", "total"};
+                                              "store", "sync_wait", "total"};
     return (i >= 0 && i < bf::N_PHASES) ? names[i] : "";
 }
 

@@ -2,6 +2,8 @@
 // translation unit per kernel variant so the variants compile in parallel.
 #pragma once
 
+#include <atomic>
+
 #include "bf_device.hip.h"
 
 namespace bf {
@@ -638,13 +640,17 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
 
 template <bool TAPS, bool PROF, bool FP8>
 hipError_t launch_variant(const KArgs& k, int grid, hipStream_t stream) {
-    // more than 64 KiB of dynamic LDS has to be requested once per kernel (per thread: cheap)
-    static thread_local bool lds_set = false;
-    if (!lds_set) {
+    // more than 64 KiB of dynamic LDS has to be requested once per kernel and device (one bit
+    // per device ordinal; a device beyond the mask asks every time)
+    static std::atomic<unsigned long long> lds_set{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return hipErrorInvalidDevice;
+    const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
+    if (!(lds_set.load(std::memory_order_relaxed) & bit)) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&eval_kernel<TAPS, PROF, FP8>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
         if (e != hipSuccess) return e;
-        lds_set = true;
+        lds_set.fetch_or(bit, std::memory_order_relaxed);
     }
     hipLaunchKernelGGL((eval_kernel<TAPS, PROF, FP8>), dim3(grid), dim3(THREADS), LDS_BYTES, stream, k);
     return hipGetLastError();

@@ -427,8 +427,8 @@ def pack_network_board(sd: Dict[str, torch.Tensor], n_layers: int, d: int, f: in
                 else:
                     sw_b[16 + i] = s_ff2[(32 * n) // BLOCK_N]
             part_b = [get(p + "norm2.weight").numpy()[own], get(p + "norm2.bias").numpy()[own],
-                      get(p + "linear1.bias").numpy()[hidden], get(p + "linear2.bias").numpy()[own],
-                      np.ascontiguousarray(wsum, dtype=np.int32).view(np.float32).reshape(-1), sw_b]
+                      get(p + "linear2.bias").numpy()[own], sw_b, get(p + "linear1.bias").numpy()[hidden],
+                      np.ascontiguousarray(wsum, dtype=np.int32).view(np.float32).reshape(-1)]
             fl += part_a + part_b
         stream.append(pack_head_tile(head, w).view(np.uint8))
         stream.append(np.zeros(8192, np.uint8))     # the weight prefetch runs one block past the end
@@ -498,6 +498,14 @@ class FusedEncoder:
         wide = self.d_model != self.D
         if wide and fp8:
             raise NotImplementedError("the 512-wide network runs in int8 only")
+        if acc_dtype == "fp32":
+            # as the reference class (brokefish/nn/cuda_impl.py:170-177): never silently dropped
+            raise NotImplementedError("acc_dtype='fp32' names an accumulator of the reference's unquantised fp16 "
+                                      "path; the quantised evaluators accumulate in int32 (int8) or fp32 (e4m3)")
+        if int8 is None and not fp8:
+            import warnings
+            warnings.warn("FusedEncoder(net) without int8=True or fp8=True builds the int8 evaluator here; the "
+                          "reference class builds its unquantised fp16 path for the same call", stacklevel=2)
         if wide and kernel in ("quad", "twin"):
             raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernels "
                                       "(kernel='octo', 'board' or 'auto') only")
@@ -529,12 +537,13 @@ class FusedEncoder:
                                ("emb_clock", 101), ("emb_rep", 3), ("policy", 64), ("promo", 4), ("value", 1)):
                 sd[name + ".weight"] = torch.zeros(rows, d)
             sd["norm_f.weight"], sd["norm_f.bias"] = torch.ones(d), torch.zeros(d)
-        # Two packings of the same weights, one per kernel (see include/brokefish_hip.h): the
-        # four-positions-per-workgroup kernel (256-wide network) and the one-position-per-workgroup
-        # kernel (int8; small launches of the 256-wide network and the 512-wide network).
+        # Two packings of the same weights (see include/brokefish_hip.h): the one-position-per-
+        # workgroup kernels (TWIN / OCTO / BOARD, what kernel="auto" runs) read the board blobs; the
+        # four-positions-per-workgroup kernel is packed, and its workspace allocated, only when it
+        # is asked for by name.
         self.kernel = kernel
         self.wstream = self.fparams = self.board_wstream = self.board_fparams = None
-        if not wide and kernel not in ("board", "twin", "octo"):
+        if kernel == "quad":
             wstream, fparams = pack_network(sd, self.n_layers, self.d_model, self.d_ff, self.n_value,
                                             fmt="e4m3" if self.fp8 else "int8")
             if wstream.size != self._lib.bf_wstream_bytes(C.byref(self._shape)) or \
@@ -542,7 +551,7 @@ class FusedEncoder:
                 raise RuntimeError("packed blob sizes disagree with the library's layout")
             self.wstream = torch.from_numpy(wstream).to(self.device)
             self.fparams = torch.from_numpy(fparams).to(self.device)
-        if kernel != "quad":
+        else:
             wstream, fparams = pack_network_board(sd, self.n_layers, self.d_model, self.d_ff, self.n_value,
                                                   fmt="e4m3" if self.fp8 else "int8")
             if wstream.size != self._lib.bf_board_wstream_bytes(C.byref(self._shape)) or \
@@ -628,7 +637,7 @@ class FusedEncoder:
         return a
 
     def kernel_choice(self, n: int) -> str:
-        """Which kernel a call with ``n`` positions runs ("quad", "board" or "twin")."""
+        """Which kernel a call with ``n`` positions runs ("quad", "board", "twin" or "octo")."""
         a = _Args()
         a.n, a.shape, a.quant, a.kernel = n, self._shape, (1 if self.fp8 else 0), self.KERNELS[self.kernel]
         a.wstream = a.fparams = 16 if self.wstream is not None else None        # only tested for NULL
@@ -743,26 +752,28 @@ class FusedEncoder:
 
     def profile_phases(self, boards, control, rep, mask=None) -> Dict[str, float]:
         """Shader-clock cycles per phase, averaged over the wavefronts of one launch of the
-        four-positions-per-workgroup kernel's profiling build (the counterpart of the
-        reference's read_profile / profile_phases).  The outputs it writes are the normal ones."""
+        profiling build of the kernel this call would run (TWIN, OCTO or QUAD, int8): the
+        counterpart of the reference's read_profile / profile_phases.  ``sync_wait`` (time at
+        workgroup barriers) is also contained in the phases around it; ``total`` is a wavefront's
+        lifetime.  The outputs it writes are the normal ones."""
         n = self._check_inputs(boards, control, rep, mask)
-        if self.wstream is None or self.fp8:
-            raise NotImplementedError("the phase profile is a build of the four-positions-per-workgroup int8 "
-                                      "kernel: construct with int8=True and kernel='auto' or 'quad'")
+        kind = self.kernel_choice(n)
+        if self.fp8 or kind == "board":
+            raise NotImplementedError("the phase profile is built for the int8 format on the TWIN, OCTO and QUAD "
+                                      "kernels (kernel='auto', 'twin', 'octo' or 'quad')")
         self._ensure_full_buffers(n)
         k = self._lib.bf_profile_phase_count()
         cyc = torch.zeros(k, dtype=torch.int64, device=self.device)
         args = self._args(boards.contiguous(), control.contiguous(), rep.contiguous(),
                           mask.contiguous() if mask is not None else None,
                           self.policy_out, self.promo_out, self.value_out, self.best_out)
-        args.kernel = self.KERNELS["quad"]
         with torch.cuda.device(self.device):
             rc = self._lib.bf_profile_phases(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
                                              C.c_void_p(cyc.data_ptr()))
         if rc:
             raise RuntimeError(f"bf_profile_phases failed ({rc}): {self._lib.bf_last_error().decode()}")
         torch.cuda.current_stream(self.device).synchronize()
-        waves = 4 * ((n + 3) // 4)
+        waves = {"twin": 4 * n, "octo": 8 * n, "quad": 4 * ((n + 3) // 4)}[kind]
         return {self._lib.bf_profile_phase_name(i).decode(): cyc[i].item() / waves for i in range(k)}
 
     # -- debug taps (the counterpart of the reference's forward_stage) ------------

@@ -218,12 +218,16 @@ double bf_mfma_rate(int quant, int* scratch, int iters, int reps, void* stream);
 
 /* In-kernel phase accounting, the counterpart of the reference's profile hooks
  * (reference csrc/encoder.cu:1083-1177 and :1886-1903: set_profile / read_profile /
- * profile_phases).  bf_profile_phases runs a separately compiled build of the evaluator
- * that reads the shader clock at phase boundaries and adds, per wavefront, the cycles of
- * each phase into cycles[bf_profile_phase_count()] (DEVICE memory, caller-zeroed).  Slot
- * "ring_wait" is the time spent waiting for weight tiles at LDS-ring synchronisations and
- * is also contained in the enclosing phases; slot "total" is the wavefront lifetime.
- * The production kernel carries none of this code. */
+ * profile_phases).  bf_profile_phases runs a separately compiled build of the kernel the
+ * arguments select (TWIN, OCTO or QUAD; int8) that reads the shader clock at phase boundaries
+ * and adds, per wavefront, the cycles of each phase into cycles[bf_profile_phase_count()]
+ * (DEVICE memory, caller-zeroed): divide by the wavefronts of the launch (TWIN 4 n, OCTO 8 n,
+ * QUAD 4 ceil(n / 4)).  Slot "sync_wait" is the time spent waiting at workgroup barriers (QUAD:
+ * at the synchronisations of the LDS weight ring) and is also contained in the enclosing phases;
+ * slot "total" is the wavefront lifetime.  In the one-position-per-workgroup kernels the matrix
+ * products of a head are issued inside "qkv_gemm_epilogue" and those of the out-projection and
+ * feed-forward tiles inside their phases; "store" is the policy / promotion / value output.
+ * The production kernels carry none of this code. */
 int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_t* cycles);
 int bf_profile_phase_count(void);
 const char* bf_profile_phase_name(int i);
@@ -308,10 +312,10 @@ int bf_movegen(const uint16_t* boards, const int16_t* control, int64_t n, uint64
  * and one block of zeros (the weight prefetch reads one block past a wave's last).
  * board_fparams is, for each wave w, per layer: part A  ln1_gamma ln1_beta b_q b_k b_v b_out
  * (own channels, d/4 each) sw_q[TW] sw_k[TW] sw_v[TW] sw_out[TW] (per own tile, padded to 16);
- * part B  ln2_gamma ln2_beta (own) b_ffn1 (own hidden channels: 128 per step) b_ffn2 (own)
- * wsum[d_ff/256][d/4] (int32, own channels) sw_ffn1[4 per step, padded to 16] sw_ffn2[TW]
- * (padded to 16; in the e4m3 format sw_ffn2[TW][d_ff/256], one per own tile and k-chunk, and
- * wsum all zero); after the four waves the embedding tables and norm_f as below.
+ * part B  ln2_gamma ln2_beta b_ffn2 (own channels) sw_ffn1[4 per step, padded to 16] sw_ffn2[TW]
+ * (padded to 16; in the e4m3 format sw_ffn2[TW][d_ff/256], one per own tile and k-chunk)
+ * b_ffn1 (own hidden channels: 128 per step) wsum[d_ff/256][d/4] (int32, own channels; all zero
+ * in the e4m3 format); after the four waves the embedding tables and norm_f as below.
  *
  * fparams (fp32 unless noted), per layer at stride bf_layer_stride_floats() (the layer's
  * parameters zero-padded to a multiple of 4 KiB, because a workgroup copies them to LDS

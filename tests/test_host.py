@@ -157,13 +157,18 @@ def test_board_packing_layout_and_sizes():
         assert (sl[:cw] == sd["encoder.layers.1.norm1.weight"].numpy()[own]).all()
         assert (sl[4 * cw:5 * cw] == sd["encoder.layers.1.self_attn.in_proj_bias"].numpy()[2 * d:][own]).all()
         assert sl[6 * cw + 2 * tw] == s_qkv[(2 * d + 32 * 2 * tw) // 128]            # sw_v of its first head
+        # part B: ln2 gamma, ln2 beta, b_ffn2, 32 weight scales, then b_ffn1 and 128 * sum(w)
         pb = sl[a_floats:]
+        assert (pb[:cw] == sd["encoder.layers.1.norm2.weight"].numpy()[own]).all()
+        assert (pb[2 * cw:3 * cw] == sd["encoder.layers.1.linear2.bias"].numpy()[own]).all()
+        assert pb[3 * cw + 5] == s_ff1[(512 + 256 + 32) // 128]                      # step 1, its second hidden tile
+        assert pb[3 * cw + 16 + 1] == s_ff2[(32 * (2 * tw + 1)) // 128]
         b1 = sd["encoder.layers.1.linear1.bias"].numpy()
-        assert (pb[2 * cw:2 * cw + 128] == b1[256:384]).all() and (pb[2 * cw + 128:2 * cw + 256] == b1[768:896]).all()
-        wsum = pb[3 * cw + 128 * steps:][: (f // 256) * cw].view(np.int32).reshape(f // 256, cw)
+        t0 = 3 * cw + 32
+        assert (pb[t0:t0 + 128] == b1[256:384]).all() and (pb[t0 + 128:t0 + 256] == b1[768:896]).all()
+        wsum = pb[t0 + 128 * steps:][: (f // 256) * cw].view(np.int32).reshape(f // 256, cw)
         assert (wsum[3] == 128 * q_ff2[own, 768:1024].astype(np.int32).sum(1)).all()
-        assert pb[b_floats - 32 + 5] == s_ff1[(512 + 256 + 32) // 128]               # step 1, its second hidden tile
-        assert pb[b_floats - 32 + 16 + 1] == s_ff2[(32 * (2 * tw + 1)) // 128]
+        assert pb.size == b_floats
         tail = fp[4 * layers * pw:]
         assert (tail[:64 * d] == sd["emb_square.weight"].numpy().reshape(-1)).all() and tail.size == (64 + 12 + 4 + 101 + 3 + 2) * d
 

@@ -288,21 +288,22 @@ def test_matrix_pipe_probe_reports_a_plausible_rate():
         assert 1000.0 < rate < 5500.0, (fmt, rate)
 
 
-def test_phase_profile_runs_the_quad_build_and_leaves_the_outputs_right():
+@pytest.mark.parametrize("kernel,n", [("auto", 64), ("auto", 1000), ("quad", 64)])
+def test_phase_profile_runs_on_the_kernel_the_call_selects_and_leaves_the_outputs_right(kernel, n):
     torch.manual_seed(0)
     net = BrokefishNet().eval()
-    model = encoder_impl("hip")(net, int8=True)               # kernel="auto": both packings present
-    b, c, r, m = positions.random_positions(64, plies=120, seed=5)
+    model = encoder_impl("hip")(net, int8=True, kernel=kernel)
+    b, c, r, m = positions.random_positions(n, plies=120, seed=5)
     bd, cd, rd, md = (t.cuda() for t in (b, c, r, m))
     want = [t.clone() for t in model.forward_full(bd, cd, rd, md)]
     for t in (model.policy_out, model.promo_out, model.value_out):
         t.zero_()
     ph = model.profile_phases(bd, cd, rd, md)
-    assert set(ph) >= {"embed", "attention", "ffn1", "ffn2", "heads", "ring_wait", "total"}
+    assert set(ph) >= {"embed", "attention", "ffn1", "ffn2", "heads", "sync_wait", "total"}
     assert all(v >= 0 for v in ph.values()) and ph["total"] > 0
-    parts = sum(v for k, v in ph.items() if k not in ("ring_wait", "total"))
+    parts = sum(v for k, v in ph.items() if k not in ("sync_wait", "total"))
     assert 0.9 * ph["total"] <= parts <= 1.0001 * ph["total"], ph   # the phases tile the wavefront's life
     for got, w in zip((model.policy_out, model.promo_out, model.value_out), want):
         assert torch.equal(got, w)
     with pytest.raises(NotImplementedError):
-        encoder_impl("hip")(net, int8=True, kernel="twin").profile_phases(bd, cd, rd, md)
+        encoder_impl("hip")(net, int8=True, kernel="board").profile_phases(bd, cd, rd, md)
