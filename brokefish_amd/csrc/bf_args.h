@@ -112,6 +112,7 @@ struct KArgs {
     float* value;
     int* best;
     int out_fp32, n_layers, l0, l1, n_value;
+    int vmode;                    // value head: 0 king row, 1 pooled (mean of the normalised live tokens), 2 prenorm
     float eps;
     float* xpark;                 // workspace: 32 KiB per board slot, residual stream parked during the FFN
     unsigned long long* profile;  // [N_PHASES] cycle sums over waves, profile builds only

@@ -317,6 +317,12 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
         (void)src;
 #pragma unroll
         for (int s = 0; s < 4; s++) asm volatile("" : "=v"(frt[set][s]));
+#elif defined(BF_EXP_HALFLOAD)   // timing experiment: half of the weight traffic
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            if (s & 1) asm volatile("" : "=v"(frt[set][s]));
+            else frt[set][s] = *reinterpret_cast<const v4i*>(src + s * FRAG);
+        }
 #else
 #pragma unroll
         for (int s = 0; s < 4; s++) frt[set][s] = *reinterpret_cast<const v4i*>(src + s * FRAG);
@@ -1139,21 +1145,18 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     }
 
     BF_PHASE(PH_HEADS);
-    // value: king token of the side to move, lane half 1 of head tile 2 holds rows 68..70
+    // raw value logits (registers 0..2 of a lane of head tile 2's upper half) to the value in [-1, 1]
+    auto value_of = [&](const v16f& hd) -> float {
+        if (a.n_value == 1) return tanh_dev(hd[0]);
+        const float r0 = hd[0], r1 = hd[1], r2 = hd[2];   // classes loss, draw, win
+        const float mx = __builtin_fmaxf(__builtin_fmaxf(r0, r1), r2);
+        const float e0 = exp_neg(r0 - mx), e1 = exp_neg(r1 - mx), e2 = exp_neg(r2 - mx);
+        return (e2 - e0) / ((e0 + e1) + e2);
+    };
+    // value (king head): king token of the side to move, lane half 1 of head tile 2 holds rows 68..70
     if (heads_here && q == 2) {
         const int king = ctrl < 0 ? 31 : 15;
-        if (lane == 32 + king) {
-            float v;
-            if (a.n_value == 1) {
-                v = tanh_dev(head[0]);
-            } else {
-                const float r0 = head[0], r1 = head[1], r2 = head[2];
-                const float mx = __builtin_fmaxf(__builtin_fmaxf(r0, r1), r2);
-                const float e0 = exp_neg(r0 - mx), e1 = exp_neg(r1 - mx), e2 = exp_neg(r2 - mx);
-                v = (e2 - e0) / ((e0 + e1) + e2);
-            }
-            a.value[b] = v;
-        }
+        if (a.vmode == 0 && lane == 32 + king) a.value[b] = value_of(head);
         if (g == 0) {   // promo: rows 64..67 are registers 0..3 of lane half 0
             if (a.out_fp32) {
                 const v4f v = {head[0], head[1], head[2], head[3]};
@@ -1212,6 +1215,58 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             const bool take = (oi != 0x7fffffff) && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi));
             bi = take ? oi : bi;
             a.best[b] = bi == 0x7fffffff ? -1 : bi;
+        }
+    }
+    // ---- pooled value heads (reference brokefish/nn/model.py:576-617) --------------------------------
+    // The value row is the mean over the live tokens of the normalised stream ("pooled", mode 1) or
+    // the final LayerNorm of the mean of the residual stream ("prenorm", mode 2); it goes through
+    // the value rows of head tile 2 like a token, and the result is in White's frame, so it is
+    // negated when Black is to move.  The token sum is a butterfly over the 32 lanes of a half
+    // (distances 16, 8, 4, 2, 1), which leaves the pooled row in every lane in a token row's layout.
+    if (a.vmode != 0) {
+        const bool live = (alive >> t) & 1u;
+        const float cdiv = (float)(__builtin_popcount(alive) > 0 ? __builtin_popcount(alive) : 1);
+        float pv[TWW][16], hv[TWW][16];
+#pragma unroll
+        for (int i = 0; i < TWW; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float v = live ? (a.vmode == 1 ? hn[i][r] : x[i][r]) : 0.0f;
+#pragma unroll
+                for (int d = 16; d >= 1; d >>= 1) v = v + __shfl_xor(v, d);
+                pv[i][r] = v / cdiv;
+            }
+        if (a.vmode == 2) {
+            layernorm(pv, gp + C::G_NFG + CW * q + 32 * t0, gp + C::G_NFB + CW * q + 32 * t0, hv);
+        } else {
+#pragma unroll
+            for (int i = 0; i < TWW; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) hv[i][r] = pv[i][r];
+        }
+        barrier();   // every wave has finished reading the normalised stream
+#pragma unroll
+        for (int i = 0; i < TWW; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const v4f v = {hv[i][4 * j], hv[i][4 * j + 1], hv[i][4 * j + 2], hv[i][4 * j + 3]};
+                *reinterpret_cast<v4f*>(hnb + (((TW * q + t0 + i) * 4 + j) * 64 + lane) * 4) = v;
+            }
+        barrier();
+        if (heads_here && q == 2) {
+            // head tile 2 once more, against the pooled row (every token column holds the same row);
+            // its blocks are read straight from the stream, in the same order as above
+            v16f hd = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            for (int f = 0; f < 8 * HB; f++) {
+                const v4f w = *reinterpret_cast<const v4f*>(wsrc + (size_t)hseq0 * BLOCK + (size_t)f * FRAG);
+                const v4f hvv = *reinterpret_cast<const v4f*>(hnb + (f * 64 + lane) * 4);
+#pragma unroll
+                for (int k = 0; k < 4; k++) hd = __builtin_amdgcn_mfma_f32_32x32x2f32(w[k], hvv[k], hd, 0, 0, 0);
+            }
+            if (lane == 32) {
+                const float v = value_of(hd);
+                a.value[b] = ctrl > 0 ? v : -v;
+            }
         }
     }
     if constexpr (PROF) {

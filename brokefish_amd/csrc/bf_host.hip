@@ -151,6 +151,10 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
         ((uintptr_t)a->mask & 7) || ((uintptr_t)a->best_move & 3))
         return fail(BF_ERR_ARGUMENT, "boards/control/value/mask/best_move must be aligned to their element size");
     if (a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
+    if (a->value_mode < BF_VALUE_KING || a->value_mode > BF_VALUE_PRENORM)
+        return fail(BF_ERR_ARGUMENT, "value_mode must be BF_VALUE_KING, BF_VALUE_POOLED or BF_VALUE_PRENORM");
+    if (a->value_mode != BF_VALUE_KING && !board)
+        return fail(BF_ERR_UNSUPPORTED, "the pooled value heads run on the one-position-per-workgroup kernels (BOARD, TWIN, OCTO)");
     if (!board && (!a->workspace || ((uintptr_t)a->workspace & 15) || a->workspace_bytes < bf_workspace_bytes(&a->shape, a->n)))
         return fail(BF_ERR_ARGUMENT, "workspace must be 16-byte aligned and hold bf_workspace_bytes(shape, n) bytes");
     memset(k, 0, sizeof(*k));
@@ -161,6 +165,7 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     k->out_fp32 = a->out_fp32 ? 1 : 0;
     k->xpark = static_cast<float*>(a->workspace);
     k->n_layers = a->shape.n_layers; k->n_value = a->shape.n_value; k->eps = a->shape.eps;
+    k->vmode = a->value_mode;
     k->l0 = 0; k->l1 = a->shape.n_layers;
     if (a->taps) {
         k->taps = *a->taps;

@@ -67,7 +67,7 @@ class _Args(C.Structure):
                 ("best_move", C.c_void_p), ("out_fp32", C.c_int32), ("quant", C.c_int32),
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("taps", C.POINTER(_Taps)),
                 ("board_wstream", C.c_void_p), ("board_fparams", C.c_void_p), ("active", C.c_void_p),
-                ("kernel", C.c_int32)]
+                ("kernel", C.c_int32), ("value_mode", C.c_int32)]
 
 
 _lib = None
@@ -451,6 +451,7 @@ class FusedEncoder:
     SHAPES = ((256, 1024, 8), (512, 2048, 16))     # (d_model, d_ff, heads) the library carries
     KERNELS = {"auto": 0, "quad": 1, "board": 2, "twin": 3, "octo": 4}   # enum bf_kernel
     ACC_DTYPES = ("fp16", "fp32")
+    VALUE_HEADS = ("king", "pooled", "prenorm")     # brokefish/nn/model.py:89
     n_value = 1
     vmode = 0
     rj_mode = 0
@@ -479,10 +480,16 @@ class FusedEncoder:
         net = source if hasattr(source, "encoder") and hasattr(source, "policy") else None
         if net is None and not hasattr(source, "layers"):
             raise ValueError("source must be a BrokefishNet or an nn.TransformerEncoder stack")
-        if net is not None and (getattr(net, "value_head", "king") != "king"
-                                or getattr(net, "reinject", "none") != "none"
-                                or getattr(net, "rule_features", False)):
-            raise NotImplementedError("only the king value head without re-injection or rule features")
+        if net is not None and (getattr(net, "reinject", "none") != "none" or getattr(net, "rule_features", False)):
+            raise NotImplementedError("re-injection and rule features are not carried by this evaluator")
+        value_head = getattr(net, "value_head", "king") if net is not None else "king"
+        if value_head not in self.VALUE_HEADS:
+            raise ValueError(f"value_head must be one of {self.VALUE_HEADS}, got {value_head!r}")
+        if value_head != "king" and kernel == "quad":
+            raise NotImplementedError("the pooled value heads run on the one-position-per-workgroup kernels "
+                                      "(kernel='auto', 'twin', 'octo' or 'board')")
+        # numbering of the reference class (brokefish/nn/cuda_impl.py:141-158): 0 king, 1 pooled, 2 prenorm
+        self.value_head, self.vmode = value_head, self.VALUE_HEADS.index(value_head)
         layers = (net.encoder if net is not None else source).layers
         first = layers[0]
         self.n_layers = len(layers)
@@ -624,6 +631,7 @@ class FusedEncoder:
         if self.board_wstream is not None:
             a.board_wstream, a.board_fparams = self.board_wstream.data_ptr(), self.board_fparams.data_ptr()
         a.kernel = self.KERNELS[self.kernel]
+        a.value_mode = self.vmode
         a.policy, a.promo, a.value = policy.data_ptr(), promo.data_ptr(), value.data_ptr()
         a.best_move = best.data_ptr() if (best is not None and mask is not None) else None
         a.out_fp32 = 1 if policy.dtype is torch.float32 else 0

@@ -7,8 +7,8 @@ model (brokefish/nn/model.py:276-361): five embedding tables, a pre-norm ReLU
 final LayerNorm, and three biasless heads; embeddings and heads N(0, 1/sqrt(d)).
 
 The evaluator only *reads* parameters from it (``FusedEncoder(net)`` snapshots them).
-Only the king value head and no re-injection / rule features are carried: those are the
-defaults every published number of the reference uses.
+The three value heads (king row, pooled, prenorm) are carried; re-injection and rule
+features are not (the defaults every published number of the reference uses).
 """
 from __future__ import annotations
 
@@ -28,9 +28,10 @@ class BrokefishNet(nn.Module):
         super().__init__()
         if n_value not in (1, 3):
             raise ValueError(f"n_value must be 1 (scalar tanh) or 3 (win/draw/loss), got {n_value}")
-        if value_head != "king" or reinject != "none" or rule_features:
-            raise NotImplementedError(
-                "only the king value head without re-injection or rule features is carried")
+        if value_head not in VALUE_HEADS:
+            raise ValueError(f"value_head must be one of {VALUE_HEADS}, got {value_head!r}")
+        if reinject != "none" or rule_features:
+            raise NotImplementedError("re-injection and rule features are not carried")
         self.d_model, self.n_layers, self.n_value = d_model, n_layers, n_value
         self.value_head, self.reinject, self.rule_features = value_head, reinject, False
         self.emb_square = nn.Embedding(N_SQUARE, d_model)
@@ -47,6 +48,10 @@ class BrokefishNet(nn.Module):
         self.policy = nn.Linear(d_model, N_POLICY, bias=False)
         self.promo = nn.Linear(d_model, N_PROMO, bias=False)
         self.value = nn.Linear(d_model, n_value, bias=False)
+        # the marker rides in the state_dict only for the pooled heads: its absence is the king
+        # head of every older checkpoint (brokefish/nn/model.py:318-331)
+        if value_head in VALUE_MODE_ID:
+            self.register_buffer("value_mode", torch.tensor(VALUE_MODE_ID[value_head], dtype=torch.int64))
         std = d_model ** -0.5
         for mod in (self.emb_square, self.emb_type_special, self.emb_color_turn, self.emb_clock,
                     self.emb_rep, self.policy, self.promo, self.value):
@@ -80,6 +85,7 @@ class BrokefishNet(nn.Module):
 # Checkpoints are bare state_dicts; what a file was trained with is recovered from the shape of
 # `value.weight` and from optional marker buffers whose absence is the legacy answer.
 
+VALUE_HEADS = ("king", "pooled", "prenorm")      # brokefish/nn/model.py:89
 VALUE_MODE_ID = {"pooled": 1, "prenorm": 2}      # brokefish/nn/model.py:93
 REINJECT_MODE_ID = {"ln1": 1, "both": 2}         # brokefish/nn/model.py:115
 RULE_FEATURES_ID = 1                             # brokefish/nn/model.py:153

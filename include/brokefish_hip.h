@@ -65,6 +65,12 @@ enum bf_kernel {
     BF_KERNEL_OCTO = 4
 };
 
+enum bf_value_mode {
+    BF_VALUE_KING = 0,
+    BF_VALUE_POOLED = 1,
+    BF_VALUE_PRENORM = 2
+};
+
 /* Sizes of one 32-token position, fixed by the position format
  * (reference docs/reference/spec.md:94-106). */
 #define BF_TOKENS 32
@@ -160,6 +166,12 @@ typedef struct {
     int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: OCTO for
                              * n <= bf_board_max_n() and for the 512-wide network, TWIN
                              * above; without the board blobs QUAD */
+    /* which tokens the value rows read (reference brokefish/nn/model.py:551-617): the king of the
+     * side to move (BF_VALUE_KING, the default), the mean of the final-normed live tokens
+     * (BF_VALUE_POOLED), or the final norm of the mean of the live tokens' residual stream
+     * (BF_VALUE_PRENORM).  The two pooled heads predict in White's frame and the result is negated
+     * when Black is to move (control < 0).  BOARD / TWIN / OCTO kernels; QUAD carries the king head. */
+    int32_t value_mode;
 } bf_eval_args;
 
 /* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */

@@ -244,7 +244,8 @@ static float* dupf(const float* p, size_t n) {
 
 bfo_model* bfo_model_create(const bfo_config* cfg, const bfo_params* p) {
     const int d = cfg->d_model, L = cfg->n_layers, f = cfg->d_ff;
-    if (d % 256 || f % 256 || d / cfg->n_heads != 32 || (cfg->n_value != 1 && cfg->n_value != 3))
+    if (d % 256 || f % 256 || d / cfg->n_heads != 32 || (cfg->n_value != 1 && cfg->n_value != 3) ||
+        cfg->value_mode < 0 || cfg->value_mode > 2)
         return NULL;
     bfo_model* m = (bfo_model*)calloc(1, sizeof(bfo_model));
     m->cfg = *cfg;
@@ -436,7 +437,8 @@ int bfo_forward(const bfo_model* m, const uint16_t* boards, const int16_t* contr
         if (taps && taps->normed) memcpy(taps->normed + (size_t)b * T * d, y, (size_t)T * d * 4);
         /* heads: one fma chain per output in lane order */
         float raw[3] = {0, 0, 0};
-        const int king = control[b] < 0 ? 31 : 15;
+        const int vmode = m->cfg.value_mode;
+        const int king = vmode ? -1 : (control[b] < 0 ? 31 : 15);
         for (int t = 0; t < T; t++)
             for (int oo = 0; oo < 68 + nv; oo++) {
                 if (oo >= 68 && t != king) continue;
@@ -452,6 +454,43 @@ int bfo_forward(const bfo_model* m, const uint16_t* boards, const int16_t* contr
                 else if (oo < 68) promo[((size_t)b * T + t) * 4 + (oo - 64)] = a;
                 else raw[oo - 68] = a;
             }
+        if (vmode) {
+            /* pooled heads (brokefish/nn/model.py:576-617): the value row is the mean over the live
+             * tokens of the normed stream (1) or norm_f of the mean of the residual stream (2).  The
+             * token sum is a butterfly (distances 16, 8, 4, 2, 1), dead tokens count as 0; the row
+             * then goes through the value rows like a token; White's frame, so negated for Black. */
+            const float* src = vmode == 1 ? y : x;
+            float* row = tmp; /* [d], then [T][d] scratch for layernorm_rows */
+            int cnt = 0;
+            for (int t = 0; t < T; t++) cnt += (alive >> t) & 1;
+            const float cdiv = (float)(cnt > 0 ? cnt : 1);
+            for (int c = 0; c < d; c++) {
+                float v[32];
+                for (int t = 0; t < T; t++) v[t] = ((alive >> t) & 1) ? src[(size_t)t * d + c] : 0.0f;
+                for (int dist = 16; dist >= 1; dist >>= 1) {
+                    float w[32];
+                    for (int t = 0; t < T; t++) w[t] = v[t] + v[t ^ dist];
+                    memcpy(v, w, sizeof v);
+                }
+                row[c] = v[0] / cdiv;
+            }
+            if (vmode == 2) {   /* the same LayerNorm as a token row gets */
+                for (int t = 1; t < T; t++) memcpy(row + (size_t)t * d, row, (size_t)d * 4);
+                layernorm_rows(row, d, m->normf_w, m->normf_b, eps, o);
+                memcpy(row, o, (size_t)d * 4);
+            }
+            for (int k = 0; k < nv; k++) {
+                const float* w = m->head_w + (size_t)(68 + k) * d;
+                float a = 0.0f;
+                for (int nn = 0; nn < d / 32; nn++)
+                    for (int r = 0; r < 16; r++)
+                        for (int g = 0; g < 2; g++) {
+                            const int c = 32 * nn + ch(r, g);
+                            a = fmaf(w[c], row[c], a);
+                        }
+                raw[k] = a;
+            }
+        }
         if (nv == 1) {
             value[b] = bfo_tanh(raw[0]);
         } else {
@@ -460,6 +499,7 @@ int bfo_forward(const bfo_model* m, const uint16_t* boards, const int16_t* contr
             const float e0 = bfo_exp_neg(raw[0] - mx), e1 = bfo_exp_neg(raw[1] - mx), e2 = bfo_exp_neg(raw[2] - mx);
             value[b] = (e2 - e0) / ((e0 + e1) + e2);
         }
+        if (vmode && !(control[b] > 0)) value[b] = -value[b];
         if (mask) {
             int best = -1;
             float bv = -INFINITY;

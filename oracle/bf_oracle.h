@@ -10,6 +10,9 @@ extern "C" {
 typedef struct {
     int d_model, n_layers, n_heads, d_ff, n_value;
     float eps;
+    /* value head (brokefish/nn/model.py:551-617): 0 king row, 1 pooled (mean of the final-normed
+     * live tokens), 2 prenorm (final norm of the mean of the live tokens' residual stream) */
+    int value_mode;
 } bfo_config;
 
 /* fp32 parameters in state_dict layout (brokefish/nn/model.py:297-316); per-layer

@@ -28,7 +28,7 @@ def build(force: bool = False) -> str:
 
 class _Config(C.Structure):
     _fields_ = [("d_model", C.c_int), ("n_layers", C.c_int), ("n_heads", C.c_int),
-                ("d_ff", C.c_int), ("n_value", C.c_int), ("eps", C.c_float)]
+                ("d_ff", C.c_int), ("n_value", C.c_int), ("eps", C.c_float), ("value_mode", C.c_int)]
 
 
 _PARAM_FIELDS = ["emb_square", "emb_type_special", "emb_color_turn", "emb_clock", "emb_rep",
@@ -170,7 +170,9 @@ class COracle:
             "value_w": _f32(sd["value.weight"]),
         }
         self._keep = arrs
-        cfg = _Config(d, L, self.n_heads, f, self.n_value, eps)
+        # the marker buffer of the pooled heads (brokefish/nn/model.py:318-331); absent: king row
+        self.value_mode = int(sd["value_mode"]) if "value_mode" in sd else 0
+        cfg = _Config(d, L, self.n_heads, f, self.n_value, eps, self.value_mode)
         prm = _Params(**{k: v.ctypes.data for k, v in arrs.items()})
         self._h = lib().bfo_model_create(C.byref(cfg), C.byref(prm))
         if not self._h:

@@ -218,6 +218,34 @@ def n_layers_of(sd) -> int:
     return n
 
 
+def value_from(sd: Dict[str, torch.Tensor], h, h_raw, control, alive, eps: float = 1e-5):
+    """The value in [-1, 1] from the side to move's point of view (brokefish/nn/model.py:551-617).
+    ``h`` is the stream after ``norm_f``, ``h_raw`` before it.  The head is the one the state_dict's
+    ``value_mode`` marker names (absent: the king row): king = the mover's king token; pooled
+    (1) = mean of the live tokens of ``h``; prenorm (2) = ``norm_f`` of the mean of the live tokens
+    of ``h_raw``.  The pooled heads predict in White's frame and are negated for Black to move."""
+    n, d = h.shape[0], h.shape[-1]
+    vmode = int(sd["value_mode"]) if "value_mode" in sd else 0
+    if vmode == 2:
+        m = alive.unsqueeze(-1).to(h_raw.dtype)
+        hv = F.layer_norm((h_raw * m).sum(1) / m.sum(1).clamp(min=1), (d,), sd["norm_f.weight"], sd["norm_f.bias"], eps)
+    elif vmode == 1:
+        m = alive.unsqueeze(-1).to(h.dtype)
+        hv = (h * m).sum(1) / m.sum(1).clamp(min=1)
+    else:
+        king = torch.where(control < 0, KING_BLACK, KING_WHITE).to(torch.int64)
+        hv = h[torch.arange(n), king]
+    raw = F.linear(hv, sd["value.weight"]).float()
+    if raw.shape[-1] == 1:
+        value = torch.tanh(raw).squeeze(-1)
+    else:  # classes 0 = loss, 1 = draw, 2 = win (brokefish/nn/model.py:156-170)
+        pr = torch.softmax(raw, dim=-1)
+        value = pr[:, 2] - pr[:, 0]
+    if vmode:
+        value = torch.where(control > 0, value, -value)
+    return value
+
+
 def forward(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8",
             mask: Optional[torch.Tensor] = None, n_heads: Optional[int] = None,
             eps: float = 1e-5, taps: Optional[dict] = None,
@@ -265,13 +293,7 @@ def forward(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8
         taps["normed"] = h.clone()
     policy = F.linear(h, sd["policy.weight"])
     promo = F.linear(h, sd["promo.weight"])
-    king = torch.where(control < 0, KING_BLACK, KING_WHITE).to(torch.int64)
-    raw = F.linear(h[torch.arange(n), king], sd["value.weight"]).float()
-    if raw.shape[-1] == 1:
-        value = torch.tanh(raw).squeeze(-1)
-    else:  # classes 0 = loss, 1 = draw, 2 = win from the side to move
-        pr = torch.softmax(raw, dim=-1)
-        value = pr[:, 2] - pr[:, 0]
+    value = value_from(sd, h, x, control, alive, eps)
     if mask is None:
         return policy, promo, value
     legal = ((mask.to(torch.int64)[..., None] >> torch.arange(64)) & 1).bool()
@@ -335,15 +357,8 @@ def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mod
         torch.backends.mha.set_fastpath_enabled(fast)
     if mode != "fp32" and hits[0] != 4 * n_layers:
         raise AssertionError(f"{hits[0]} matmuls were diverted, expected {4 * n_layers}")
-    h = F.layer_norm(h, (d,), sd["norm_f.weight"], sd["norm_f.bias"], eps)
+    h_raw = h
+    h = F.layer_norm(h_raw, (d,), sd["norm_f.weight"], sd["norm_f.bias"], eps)
     policy = plain_linear(h, sd["policy.weight"])
     promo = plain_linear(h, sd["promo.weight"])
-    n = x.shape[0]
-    king = torch.where(control < 0, KING_BLACK, KING_WHITE).to(torch.int64)
-    raw = plain_linear(h[torch.arange(n), king], sd["value.weight"]).float()
-    if raw.shape[-1] == 1:
-        value = torch.tanh(raw).squeeze(-1)
-    else:
-        pr = torch.softmax(raw, dim=-1)
-        value = pr[:, 2] - pr[:, 0]
-    return policy, promo, value
+    return policy, promo, value_from(sd, h, h_raw, control, alive, eps)

@@ -25,6 +25,17 @@ What it records, and why these need the reference itself rather than a closed fo
   ``emulated_forward(net, QuantConfig(weights=True, activations=True, q_max=8, tile_k=256))``.
   torch's fp32 matmul fixes the summation order inside a k-tile, which no closed form gives.
 
+* (third file, ``python tests/golden/make_golden.py layers``) what the reference's own
+  ``emulated_forward`` holds **inside** the golden int8 network, for positions 0-1 and layers 0, 3
+  and 7: the residual stream entering the layer, and for each of the four patched matmuls the
+  operand bytes and activation scales of ``quantise_activations_int8`` on the tensor the patch
+  received, and the exact integer accumulators per 256-deep k-chunk of
+  ``int8_linear`` (quant.py:299-301: the product of those operands with
+  ``quantise_weights_int8_bytes`` of the module's weight) -- in full for position 0 at layer 0,
+  as position-weighted row checksums elsewhere; the layer's output for position 0.  And the
+  value of the pooled / prenorm value heads (model.py:576-617), 1 and 3 value rows, in fp32 and
+  int8-simulated, on the eight positions.
+
 Inputs are regenerated from the formulas below by the tests; only outputs are stored.
 """
 from __future__ import annotations
@@ -176,5 +187,96 @@ def main() -> int:
     return 0
 
 
+LAYER_TAPS = (0, 3, 7)
+MATMUL_OF = {"qkv": "self_attn.in_proj_weight", "out": "self_attn.out_proj.weight",
+             "ff1": "linear1.weight", "ff2": "linear2.weight"}
+
+
+def row_checksum(acc: np.ndarray) -> np.ndarray:
+    """[..., N] integer accumulators -> [...] int64: sum over the output channel n of acc * (n % 1009 + 1)."""
+    w = (np.arange(acc.shape[-1], dtype=np.int64) % 1009) + 1
+    return (acc.astype(np.int64) * w).sum(axis=-1)
+
+
+def main_layers() -> int:
+    sys.path.insert(0, REFERENCE)
+    from brokefish.nn import quant as rq                      # noqa: E402
+    from brokefish.nn.model import BrokefishNet as RefNet     # noqa: E402
+
+    out = {}
+    torch.manual_seed(0)
+    net = RefNet(n_value=1).eval()
+    net.load_state_dict(fill_state_dict(net.state_dict()))
+    boards, control, rep = positions()
+    boards, control, rep = boards[:2], control[:2], rep[:2]
+    which = {}
+    for l in LAYER_TAPS:
+        lay = net.encoder.layers[l]
+        which[id(lay.self_attn.in_proj_weight)] = (l, "qkv")
+        which[id(lay.self_attn.out_proj.weight)] = (l, "out")
+        which[id(lay.linear1.weight)] = (l, "ff1")
+        which[id(lay.linear2.weight)] = (l, "ff2")
+    original = rq.int8_linear
+
+    def recording(x, w, bias, unsigned=False, row_k=rq.ROW_K):
+        tag = which.get(id(w))
+        if tag is not None:
+            l, name = tag
+            a = x.reshape(-1, x.shape[-1]).float()
+            wq, ws = rq.quantise_weights_int8_bytes(w.float())
+            wq = wq.view(torch.int8).double()
+            qs, sas, accs = [], [], []
+            for lo in range(0, a.shape[1], row_k):
+                tq, sa = rq.quantise_activations_int8(a[:, lo:lo + row_k], unsigned)
+                qs.append(tq)
+                sas.append(sa)
+                accs.append((tq.double() @ wq[:, lo:lo + row_k].T).round().to(torch.int64))
+            q = torch.cat(qs, dim=1).reshape(2, 32, -1)
+            acc = torch.stack(accs).reshape(len(accs), 2, 32, -1).numpy()          # [kc, 2, 32, N]
+            assert np.abs(acc).max() < 2 ** 31
+            key = f"l{l}_{name}"
+            out[f"qa_{key}"] = q.numpy().astype(np.uint8 if unsigned else np.int8)
+            out[f"sa_{key}"] = torch.cat(sas, dim=1).reshape(2, 32, -1).numpy()
+            out[f"accsum_{key}"] = row_checksum(acc)                              # [kc, 2, 32]
+            if l == LAYER_TAPS[0]:
+                out[f"acc_{key}"] = acc[:, 0].astype(np.int32)                    # position 0 in full
+        return original(x, w, bias, unsigned=unsigned, row_k=row_k)
+
+    hooks = []
+    for l in LAYER_TAPS:
+        hooks.append(net.encoder.layers[l].register_forward_pre_hook(
+            lambda m, args, l=l: out.__setitem__(f"x_in_l{l}", args[0].detach().clone().numpy())))
+        hooks.append(net.encoder.layers[l].register_forward_hook(
+            lambda m, args, o, l=l: out.__setitem__(f"x_out_l{l}", o.detach()[:1].clone().numpy())))
+    rq.int8_linear = recording
+    try:
+        with torch.no_grad():
+            p8, q8, v8 = rq.emulated_forward(net, rq.QuantConfig(fmt="int8"))(boards, control, rep)
+    finally:
+        rq.int8_linear = original
+        for h in hooks:
+            h.remove()
+    out["int8_policy_2"], out["int8_value_2"] = p8.numpy(), v8.numpy()
+
+    # the pooled value heads: same formula weights (the marker buffer is not a float tensor and
+    # sorts after every float key), so policy and promotion logits are those of the king net
+    boards, control, rep = positions()
+    for head in ("pooled", "prenorm"):
+        for n_value in (1, 3):
+            torch.manual_seed(0)
+            vnet = RefNet(n_value=n_value, value_head=head).eval()
+            vnet.load_state_dict(fill_state_dict(vnet.state_dict()))
+            with torch.no_grad():
+                p32, q32, v32 = vnet(boards, control, rep)
+                p8, q8, v8 = rq.emulated_forward(vnet, rq.QuantConfig(fmt="int8"))(boards, control, rep)
+            out[f"fp32_value_{head}_nv{n_value}"], out[f"int8_value_{head}_nv{n_value}"] = v32.numpy(), v8.numpy()
+            out[f"int8_policysum_{head}_nv{n_value}"] = np.array(p8.double().sum().item())
+    out["torch_version"] = np.array(torch.__version__)
+    path = os.path.join(HERE, "reference_vectors_layers.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, {k: getattr(v, "shape", None) for k, v in out.items()}, os.path.getsize(path), "bytes")
+    return 0
+
+
 if __name__ == "__main__":
-    raise SystemExit(main())
+    raise SystemExit(main_layers() if sys.argv[1:] == ["layers"] else main())

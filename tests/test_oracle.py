@@ -356,6 +356,77 @@ def test_value_head_rules():
     assert np.abs(o1["value"] - np.tanh(raw1)).max() < 1e-5
 
 
+@pytest.fixture(scope="module")
+def golden_layers():
+    import os
+    return np.load(os.path.join(os.path.dirname(mg.__file__), "reference_vectors_layers.npz"))
+
+
+def _golden_value_net(head, nv):
+    torch.manual_seed(0)
+    net = BrokefishNet(n_value=nv, value_head=head).eval()
+    sd = mg.fill_state_dict(net.state_dict())
+    return (sd,) + tuple(mg.positions())
+
+
+@pytest.mark.parametrize("head", ["pooled", "prenorm"])
+@pytest.mark.parametrize("nv", [1, 3])
+def test_pooled_value_heads_against_the_reference(golden, golden_layers, head, nv):
+    # the reference's own model with value_head="pooled" / "prenorm" (brokefish/nn/model.py:576-617;
+    # its tests: tests/test_b2.py:520-650) wrote these values for the formula weights
+    sd, b, c, r = _golden_value_net(head, nv)
+    assert int(sd["value_mode"]) == {"pooled": 1, "prenorm": 2}[head]
+    with torch.no_grad():
+        got32 = emulated.forward(sd, b, c, r, mode="fp32")
+    assert np.abs(got32[2].numpy() - golden_layers[f"fp32_value_{head}_nv{nv}"]).max() < 2e-6
+    got8 = emulated.forward_library_stack(sd, b, c, r, mode="int8")
+    if str(golden_layers["torch_version"]) == torch.__version__:
+        assert (got8[2].numpy().view(np.int32) == golden_layers[f"int8_value_{head}_nv{nv}"].view(np.int32)).all()
+        assert abs(got8[0].double().sum().item() - float(golden_layers[f"int8_policysum_{head}_nv{nv}"])) < 1e-9
+    # the head changes the value only: the logits are the king net's
+    nb = 3 if nv == 3 else 8
+    assert np.abs(got32[0].numpy()[:nb] - golden[f"fp32_policy_nv{nv}"]).max() < 2e-5
+    assert not np.allclose(got32[2].numpy()[:nb], golden[f"fp32_value_nv{nv}"], atol=1e-3)
+
+
+@pytest.mark.parametrize("head", ["pooled", "prenorm"])
+@pytest.mark.parametrize("nv", [1, 3])
+def test_c_checker_pooled_value_heads_teacher_forced(head, nv):
+    # the C checker's pooled heads (butterfly token sum, the token LayerNorm on the pooled row, the
+    # value rows' fma chain, negation for Black) given the same residual stream as the torch
+    # restatement: agreement to fp32 rounding, both colours, dead slots excluded from the mean
+    torch.manual_seed(5)
+    net = BrokefishNet(n_value=nv, value_head=head, n_layers=2).eval().randomise_layers_(seed=9)
+    sd = {k: v.detach() for k, v in net.state_dict().items()}
+    b, c, r, _ = positions.random_positions(48, plies=120, seed=7)
+    assert (c < 0).any() and (c > 0).any()
+    taps = {}
+    with torch.no_grad():
+        want = emulated.forward(sd, b, c, r, mode="int8", taps=taps)
+    x_last = taps["resid"][-1].numpy()
+    co = c_oracle.COracle(sd)
+    assert co.value_mode == {"pooled": 1, "prenorm": 2}[head]
+    got = co.forward(b.numpy(), c.numpy(), r.numpy(), x_in=x_last, layer_begin=2, layer_end=2)
+    assert np.abs(got["value"] - want[2].numpy()).max() < 2e-6
+    # closed form in float64 from the checker's own normed / residual stream
+    alive = ((b.numpy().view(np.uint16) >> 11) & 1) == 0
+    full = co.forward(b.numpy(), c.numpy(), r.numpy(), taps=True)
+    src = full["normed"] if head == "pooled" else full["resid"][:, -1]
+    pooled = (src.astype(np.float64) * alive[..., None]).sum(1) / np.maximum(alive.sum(1), 1)[:, None]
+    if head == "prenorm":
+        mu, var = pooled.mean(1, keepdims=True), pooled.var(1, keepdims=True)
+        pooled = (pooled - mu) / np.sqrt(var + 1e-5) * sd["norm_f.weight"].numpy() + sd["norm_f.bias"].numpy()
+    raw = pooled @ sd["value.weight"].numpy().astype(np.float64).T
+    if nv == 1:
+        val = np.tanh(raw[:, 0])
+    else:
+        p = np.exp(raw - raw.max(1, keepdims=True))
+        p /= p.sum(1, keepdims=True)
+        val = p[:, 2] - p[:, 0]
+    val = np.where(c.numpy() > 0, val, -val)
+    assert np.abs(full["value"] - val).max() < 2e-6
+
+
 def test_mask_and_argmax_closed_form():
     net, sd = _net()
     co = c_oracle.COracle(sd)

@@ -279,6 +279,39 @@ def test_stress_network_win_draw_loss_head_and_full_batch_properties():
     assert torch.gather(legal.reshape(n, -1)[has], 1, best[has].long()[:, None]).all()
 
 
+@pytest.mark.parametrize("head", ["pooled", "prenorm"])
+@pytest.mark.parametrize("nv", [1, 3])
+def test_pooled_value_heads_bit_exact_on_every_kernel(head, nv):
+    # reference brokefish/nn/model.py:576-617 (its tests: tests/test_b2.py:520-650): the value row is
+    # the mean of the live tokens (after or before norm_f) and the result is negated for Black
+    torch.manual_seed(1)
+    net = BrokefishNet(n_value=nv, value_head=head).eval().randomise_layers_(seed=4)
+    sd = {k: v.detach() for k, v in net.state_dict().items()}
+    b, c, r, m = positions.random_positions(96, plies=120, seed=13, stamp_queen=True)
+    assert (c < 0).any() and (c > 0).any()
+    want = c_oracle.COracle(sd).forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy())
+    bd, cd, rd, md = _dev(b, c, r, m)
+    for kernel in ("twin", "octo", "board", "auto"):
+        model = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=kernel)
+        assert model.vmode == {"pooled": 1, "prenorm": 2}[head]
+        p, q, v, best = model.forward_masked(bd, cd, rd, md)
+        assert _bits_equal(v, want["value"]), (kernel, np.abs(v.cpu().numpy() - want["value"]).max())
+        assert _bits_equal(p, want["policy"]) and _bits_equal(q, want["promo"]) and (best.cpu().numpy() == want["best"]).all()
+    # the king head of the same weights gives other values; the sign flip shows on a colour swap of the control word
+    king = BrokefishNet(n_value=nv).eval()
+    king.load_state_dict({k: v for k, v in sd.items() if k != "value_mode"})
+    vk = encoder_impl("hip")(king, int8=True, out_dtype=torch.float32).forward_full(bd, cd, rd)[2]
+    assert not torch.allclose(vk, v, atol=1e-3)
+    with pytest.raises(NotImplementedError):
+        encoder_impl("hip")(net, int8=True, kernel="quad")
+    wide = BrokefishNet(d_model=512, n_heads=16, d_ff=2048, n_layers=2, n_value=nv, value_head=head).eval().randomise_layers_(seed=6)
+    sdw = {k: v.detach() for k, v in wide.state_dict().items()}
+    ww = c_oracle.COracle(sdw).forward(b.numpy()[:24], c.numpy()[:24], r.numpy()[:24])
+    for kernel in ("octo", "board"):
+        vw = encoder_impl("hip")(wide, int8=True, out_dtype=torch.float32, kernel=kernel).forward_full(bd[:24], cd[:24], rd[:24])[2]
+        assert _bits_equal(vw, ww["value"]), kernel
+
+
 def test_matrix_pipe_probe_reports_a_plausible_rate():
     # a register-resident MFMA loop cannot beat the datasheet peak (5.0 POP/s dense int8 / fp8)
     # and, on a healthy part, reaches most of it; the evaluator's own rate must lie below it
