@@ -231,12 +231,19 @@ def main_layers() -> int:
                 qs.append(tq)
                 sas.append(sa)
                 accs.append((tq.double() @ wq[:, lo:lo + row_k].T).round().to(torch.int64))
-            q = torch.cat(qs, dim=1).reshape(2, 32, -1)
-            acc = torch.stack(accs).reshape(len(accs), 2, 32, -1).numpy()          # [kc, 2, 32, N]
+            # rows arrive as (position, token) outside the attention module and as (token, position)
+            # inside it (torch's multi_head_attention_forward works on [T, B, E])
+            inside = name in ("qkv", "out")
+
+            def by_position(t):      # [rows, C] -> [2, 32, C]
+                return t.reshape(32, 2, -1).transpose(0, 1) if inside else t.reshape(2, 32, -1)
+
+            q = by_position(torch.cat(qs, dim=1))
+            acc = torch.stack([by_position(a_) for a_ in accs]).numpy()            # [kc, 2, 32, N]
             assert np.abs(acc).max() < 2 ** 31
             key = f"l{l}_{name}"
             out[f"qa_{key}"] = q.numpy().astype(np.uint8 if unsigned else np.int8)
-            out[f"sa_{key}"] = torch.cat(sas, dim=1).reshape(2, 32, -1).numpy()
+            out[f"sa_{key}"] = by_position(torch.cat(sas, dim=1)).numpy()
             out[f"accsum_{key}"] = row_checksum(acc)                              # [kc, 2, 32]
             if l == LAYER_TAPS[0]:
                 out[f"acc_{key}"] = acc[:, 0].astype(np.int32)                    # position 0 in full

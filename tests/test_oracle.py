@@ -427,6 +427,24 @@ def test_c_checker_pooled_value_heads_teacher_forced(head, nv):
     assert np.abs(full["value"] - val).max() < 2e-6
 
 
+def test_c_checker_layer_by_layer_from_the_references_own_residual_stream(capsys):
+    # The reference's emulated_forward wrote, for layers 0, 3, 7 of the golden network, the residual
+    # stream entering the layer and every operand byte, scale and int32 accumulator inside it
+    # (tests/golden/make_golden.py `layers`).  The C checker, run on that one layer from the
+    # reference's stream, must give the reference's bytes (but for provable rounding ties) and the
+    # reference's accumulators exactly.
+    import reflayers
+    _, _, sd, b, c, r = reflayers.load()
+    co = c_oracle.COracle(sd)
+
+    def run_layer(l, x_in):
+        return co.forward(b.numpy(), c.numpy(), r.numpy(), taps=True, x_in=x_in, layer_begin=l, layer_end=l + 1)
+
+    stats = reflayers.check(run_layer)
+    with capsys.disabled():
+        print("\n  C checker vs the reference's per-layer data:", stats)
+
+
 def test_mask_and_argmax_closed_form():
     net, sd = _net()
     co = c_oracle.COracle(sd)
