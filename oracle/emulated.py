@@ -108,7 +108,7 @@ def int8_linear(x, w, bias, unsigned: bool = False, taps: Optional[dict] = None,
     wq, ws = quantise_weights_int8(w)
     wq64 = wq.to(torch.float64)
     out = torch.zeros(m, n, dtype=torch.float64)
-    qs, accs = [], []
+    qs, accs, quots = [], [], []
     for lo in range(0, k, ROW_K):
         q, sa = quantise_activations_int8(a[:, lo:lo + ROW_K], unsigned)
         acc = q.to(torch.float64) @ wq64[:, lo:lo + ROW_K].T
@@ -116,9 +116,13 @@ def int8_linear(x, w, bias, unsigned: bool = False, taps: Optional[dict] = None,
         if taps is not None:
             qs.append(q.to(torch.int16))
             accs.append(acc.to(torch.int32))
+            src = a[:, lo:lo + ROW_K].clamp(min=0) if unsigned else a[:, lo:lo + ROW_K]
+            quots.append(src.to(torch.float64) / sa.to(torch.float64))
     if taps is not None:
         taps.setdefault("qa_" + name, []).append(torch.cat(qs, dim=1))
         taps.setdefault("acc_" + name, []).append(torch.stack(accs))
+        # the quotients x / s before rounding, in float64: how far each byte was from a tie
+        taps.setdefault("quot_" + name, []).append(torch.cat(quots, dim=1))
     y = out.to(torch.float32) * ws.repeat_interleave(BLOCK_N)[None, :]
     if bias is not None:
         y = y + bias.float()
@@ -198,6 +202,8 @@ def fp8_linear(x, w, bias, taps: Optional[dict] = None, name: str = "", q_max: f
         taps.setdefault("qa_" + name, []).append(aq.clone())
         taps.setdefault("sa_" + name, []).append(sa.clone())
         taps.setdefault("acc_" + name, []).append(torch.stack(accs))
+        # the quotients x / s before rounding to e4m3, in float64: how far each byte was from a tie
+        taps.setdefault("quot_" + name, []).append(a.to(torch.float64) / sa.to(torch.float64).repeat_interleave(tile_k, dim=1))
     if bias is not None:
         out = out + bias.float()
     return out.reshape(*lead, n).to(x.dtype)

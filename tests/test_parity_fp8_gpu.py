@@ -29,6 +29,7 @@ import pytest
 import torch
 
 import make_golden as mg
+import reflayers
 from brokefish_amd import encoder_impl, positions
 from brokefish_amd.net import BrokefishNet
 from oracle import emulated
@@ -52,7 +53,7 @@ def _dev(*ts):
     return [t.cuda() for t in ts]
 
 
-def test_teacher_forced_layers_against_the_emulation(setup):
+def test_teacher_forced_layers_against_the_emulation(setup, capsys):
     net, sd, model = setup
     n = 32
     b, c, r, _ = positions.random_positions(n, plies=100, seed=16, stamp_queen=True)
@@ -61,6 +62,7 @@ def test_teacher_forced_layers_against_the_emulation(setup):
         ref = emulated.forward(sd, b, c, r, mode="e4m3", taps=taps)
     bd, cd, rd = _dev(b, c, r)
     x_in = taps["embed"]
+    n_flips, n_bytes, worst = 0, 0, [0.0, 0.0]
     for l in range(8):
         got = model.forward_taps(bd, cd, rd, x_in=x_in.cuda(), layer_begin=l, layer_end=l + 1)
         dirty = np.zeros((n, 32), bool)
@@ -68,13 +70,18 @@ def test_teacher_forced_layers_against_the_emulation(setup):
             qt = taps["qa_" + name][l].reshape(n, 32, -1).numpy()
             qg = got["qa_" + name][:, 0].cpu().float().numpy()
             mism = qt != qg
-            if name == "qkv":        # identical input, exact quantiser: identical bytes (ties aside)
-                assert mism.mean() < 1e-5
-            else:
-                assert mism[~dirty].mean() < 2e-5
-                # a flipped byte is the neighbouring e4m3 value: one step is at most 1/8 of the magnitude
-                first = mism & ~dirty[..., None]          # rows whose inputs were still clean
-                assert (np.abs(qt - qg)[first] <= 0.1251 * np.maximum(np.abs(qt), np.abs(qg))[first] + 2.0 ** -9).all()
+            # Every flipped byte on a row whose inputs were still clean is the neighbouring e4m3 value
+            # (one step is at most 1/8 of the magnitude) and a provable tie: the emulation's own
+            # quotient x / s (float64) sits on the midpoint of two neighbouring e4m3 values to within
+            # the distance two fp32 summation orders of the same input can differ by.
+            first = mism & ~dirty[..., None]
+            assert (np.abs(qt - qg)[first] <= 0.1251 * np.maximum(np.abs(qt), np.abs(qg))[first] + 2.0 ** -9).all()
+            dist = reflayers.e4m3_tie_distance(taps["quot_" + name][l].numpy().reshape(n, 32, -1))
+            tol = reflayers.E4M3_TIE_TOL if name == "qkv" else reflayers.E4M3_TIE_TOL_AFTER_MATMUL
+            assert (dist[first] <= tol).all(), (l, name, int(first.sum()), float(dist[first].max()))
+            n_flips += int(first.sum())
+            n_bytes += int((~dirty).sum()) * qt.shape[-1]
+            worst[name != "qkv"] = max(worst[name != "qkv"], float(dist[first].max()) if first.any() else 0.0)
             # the accumulators against the exact product of the kernel's OWN operand bytes
             wq = emulated.quantise_weights_e4m3(sd[f"encoder.layers.{l}.{WEIGHT[name]}"])[0].numpy().astype(np.float64)
             ag = got["acc_" + name][:, 0].cpu().numpy()                       # [n, kc, 32, N]
@@ -91,13 +98,17 @@ def test_teacher_forced_layers_against_the_emulation(setup):
         assert d[~dirty].max() < 1e-5 and (~dirty).mean() > 0.9
         assert d.max() < 0.5                        # a flipped byte moves a row by a bounded amount
         x_in = x_next
+    with capsys.disabled():
+        print(f"\n  e4m3 HIP vs emulation, teacher-forced: {n_flips} flipped bytes of {n_bytes} on clean rows; distance from an "
+              f"e4m3 tie at most {worst[0]:.2e} (first quantiser, allowed {reflayers.E4M3_TIE_TOL:.2e}) / {worst[1]:.2e} "
+              f"(behind a matmul, allowed {reflayers.E4M3_TIE_TOL_AFTER_MATMUL:.2e})")
     got = model.forward_taps(bd, cd, rd, x_in=taps["resid"][7].cuda(), layer_begin=8, layer_end=8, want=["normed"])
     assert (got["policy"].cpu() - ref[0]).abs().max() < 1e-4
     assert (got["promo"].cpu() - ref[1]).abs().max() < 1e-4
     assert (got["value"].cpu() - ref[2]).abs().max() < 1e-5
 
 
-def test_free_running_accuracy_equals_the_emulations(setup):
+def test_free_running_accuracy_equals_the_emulations(setup, capsys):
     net, sd, model = setup
     b, c, r, _ = positions.random_positions(64, plies=120, seed=11, stamp_queen=True)
     with torch.no_grad():
@@ -105,10 +116,39 @@ def test_free_running_accuracy_equals_the_emulations(setup):
         f32 = emulated.forward(sd, b, c, r, mode="fp32")
     got = [t.cpu() for t in model.forward_full(*_dev(b, c, r))]
     assert all(torch.isfinite(t).all() for t in got)
-    # the stated target (logits within 2e-2 of the emulation) holds on every board that saw no
-    # flipped byte: more than half of them, and half of all boards are within 1e-4
-    per_board = (got[0] - emu[0]).abs().reshape(64, -1).amax(1)
-    assert (per_board <= 2e-2).float().mean() > 0.5 and per_board.median() < 1e-4
+    # The stated target (logits within 2e-2 of the emulation) board by board: run both with taps,
+    # walk each board's quantisers in order (layer, then qkv / out / ff1 / ff2) to its FIRST
+    # diverging operand byte.  A board with none must meet the target -- every such board, not a
+    # share of them; and every first divergence must be a provable e4m3 tie (up to there the two
+    # sides computed the same numbers to fp32 summation order).
+    etaps = {}
+    with torch.no_grad():
+        emulated.forward(sd, b, c, r, mode="e4m3", taps=etaps)
+    gtaps = model.forward_taps(*_dev(b, c, r), want=["qa_qkv", "qa_out", "qa_ff1", "qa_ff2"])
+    assert torch.equal(gtaps["policy"].cpu(), got[0])
+    per_board = (got[0] - emu[0]).abs().reshape(64, -1).amax(1).numpy()
+    per_board_v = (got[2] - emu[2]).abs().numpy()
+    flipped = np.zeros(64, bool)
+    worst = 0.0
+    for l in range(8):
+        for name in ("qkv", "out", "ff1", "ff2"):
+            qt = etaps["qa_" + name][l].reshape(64, 32, -1).numpy()
+            qg = gtaps["qa_" + name][:, l].cpu().float().numpy()
+            mism = qt != qg
+            first = mism & ~flipped[:, None, None]
+            if first.any():
+                dist = reflayers.e4m3_tie_distance(etaps["quot_" + name][l].numpy().reshape(64, 32, -1))[first]
+                worst = max(worst, float(dist.max()))
+                tol = reflayers.E4M3_TIE_TOL if (l == 0 and name == "qkv") else reflayers.E4M3_TIE_TOL_AFTER_MATMUL
+                assert (dist <= tol).all(), (l, name, float(dist.max()))
+            flipped |= mism.any((1, 2))
+    with capsys.disabled():
+        print(f"\n  e4m3 free-running, 64 boards: {int((~flipped).sum())} without a flipped byte, worst of them "
+              f"{per_board[~flipped].max():.2e} from the emulation (target 2e-2); {int(flipped.sum())} with a first flip "
+              f"(a tie to {worst:.2e}), of them {(per_board[flipped] <= 2e-2).sum()} still within 2e-2, worst {per_board.max():.3f}")
+    assert (~flipped).sum() >= 16
+    assert (per_board[~flipped] <= 2e-2).all() and (per_board_v[~flipped] <= 2e-2).all()
+    assert per_board[~flipped].max() < 1e-4          # in fact they agree to fp32 rounding
     assert per_board.max() < 0.3
     for i in (0, 1, 2):
         err_kernel, err_emu = (got[i] - f32[i]).abs(), (emu[i] - f32[i]).abs()

@@ -16,6 +16,7 @@ import torch
 from brokefish_amd import encoder_impl, positions
 from brokefish_amd.net import BrokefishNet
 from oracle import c_oracle, emulated
+import reflayers
 
 pytestmark = pytest.mark.gpu
 
@@ -192,7 +193,7 @@ def test_every_clock_and_rep_and_dead_slot_inertness_on_device(nets):
     assert torch.isfinite(p2).all()
 
 
-def test_teacher_forced_layers_against_the_torch_restatement(nets):
+def test_teacher_forced_layers_against_the_torch_restatement(nets, capsys):
     net, sd, model, co = nets["distinct"]
     n = 32
     b, c, r, _ = positions.random_positions(n, plies=100, seed=16, stamp_queen=True)
@@ -201,6 +202,7 @@ def test_teacher_forced_layers_against_the_torch_restatement(nets):
         ref = emulated.forward(sd, b, c, r, mode="int8", taps=taps)
     bd, cd, rd = _dev(b, c, r)
     x_in = taps["embed"]
+    n_flips, n_bytes, worst = 0, 0, 0.0
     for l in range(8):
         got = model.forward_taps(bd, cd, rd, x_in=x_in.cuda(), layer_begin=l, layer_end=l + 1,
                                  want=TAPS_INT + ["resid"])
@@ -209,7 +211,16 @@ def test_teacher_forced_layers_against_the_torch_restatement(nets):
             qt = taps["qa_" + name][l].numpy().reshape(n, 32, -1).astype(np.int32)
             qg = got["qa_" + name][:, 0].cpu().numpy().astype(np.int32)
             mism = qt != qg
-            assert np.abs(qt - qg)[~dirty].max() <= 1 and mism[~dirty].mean() < 1e-3
+            assert np.abs(qt - qg)[~dirty].max() <= 1
+            # every flipped byte on a clean row is a provable tie: the quotient x / s (float64, from
+            # the restatement's own fp32 x and s) sits within 2^-18 of full scale of a rounding boundary
+            flips = mism & ~dirty[..., None]
+            dist = reflayers.tie_distance(taps["quot_" + name][l].numpy().reshape(n, 32, -1))
+            tol = reflayers.TIE_TOL_U8 if name == "ff2" else reflayers.TIE_TOL
+            assert (dist[flips] <= tol).all(), (l, name, int(flips.sum()), float(dist[flips].max()))
+            n_flips += int(flips.sum())
+            n_bytes += int((~dirty).sum()) * qt.shape[-1]
+            worst = max(worst, float(dist[flips].max()) if flips.any() else 0.0)
             at = taps["acc_" + name][l].numpy()
             at = at.reshape(at.shape[0], n, 32, -1).transpose(1, 2, 0, 3)           # [n,32,kc,N]
             ag = got["acc_" + name][:, 0].cpu().numpy().transpose(0, 2, 1, 3)
@@ -223,6 +234,9 @@ def test_teacher_forced_layers_against_the_torch_restatement(nets):
         assert d[~dirty].max() < 2e-5 * max(float(x_next.abs().max()), 1.0)
         assert (~dirty).mean() > 0.5
         x_in = x_next
+    with capsys.disabled():
+        print(f"\n  HIP vs torch restatement, teacher-forced: {n_flips} flipped bytes of {n_bytes} on clean rows, "
+              f"every one within {worst:.2e} steps of a tie (allowed {reflayers.TIE_TOL:.2e})")
     # heads, teacher-forced on the torch restatement's final residual stream
     got = model.forward_taps(bd, cd, rd, x_in=taps["resid"][7].cuda(), layer_begin=8, layer_end=8, want=["normed"])
     assert (got["policy"].cpu() - ref[0]).abs().max() < 1e-4            # tolerance: fp32 re-ordering, << 1e-3

@@ -90,8 +90,12 @@ def test_checkpoint_conventions_size_a_net_from_a_bare_state_dict():
     for key, val, fn in (("value_mode", 1, "pooled"), ("value_mode", 2, "prenorm")):
         marked = dict(state, **{key: torch.tensor(val)})
         assert bn.value_head_of(marked) == fn
+        dst = bn.net_for_state(marked)                     # the pooled heads are carried: the marker rides along
+        dst.load_state_dict(marked, strict=True)
+        assert dst.value_head == fn and int(dst.state_dict()["value_mode"]) == val
+    for key, val in (("reinject_mode", 1), ("rule_features_mode", 1)):
         with pytest.raises(NotImplementedError):
-            bn.net_for_state(marked)                       # recognised, and loudly not carried
+            bn.net_for_state(dict(state, **{key: torch.tensor(val)}))    # recognised, and loudly not carried
     assert bn.reinject_of(dict(state, reinject_mode=torch.tensor(2))) == "both"
     assert bn.rule_features_of(dict(state, rule_features_mode=torch.tensor(1))) is True
     with pytest.raises(ValueError):
