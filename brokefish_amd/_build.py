@@ -5,6 +5,7 @@ gfx950.  Two shared libraries live next to this file:
 
 * ``libbrokefish_hip.so``  -- the HIP kernels and the C-ABI of ``include/brokefish_hip.h``
 * ``libbf_chessgen.so``    -- the CPU rules engine that makes synthetic positions
+* ``_bf_torch.so``         -- the PyTorch extension module over that C-ABI (tensors in, current stream)
 """
 from __future__ import annotations
 
@@ -18,6 +19,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(ROOT, "include")
 HIP_LIB = os.path.join(HERE, "libbrokefish_hip.so")
 CHESSGEN_LIB = os.path.join(HERE, "libbf_chessgen.so")
+TORCH_EXT = os.path.join(HERE, "_bf_torch.so")
 
 HIP_SOURCES = ["bf_host.hip", "bf_expand.hip", "bf_movegen.hip", "bf_probe.hip", "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip",
                "bf_variant_prod_fp8.hip", "bf_variant_taps_fp8.hip",
@@ -85,6 +87,32 @@ def build_chessgen() -> str:
     return CHESSGEN_LIB
 
 
+def build_torch_ext() -> str:
+    """The PyTorch extension module brokefish_amd._bf_torch (host code only: it calls the C-ABI of
+    libbrokefish_hip.so, which must have been built).  The counterpart of the reference's
+    ``load_extension`` (brokefish/nn/_build.py:149-190), compiled in-tree with the flags
+    ``torch.utils.cpp_extension`` uses for a ROCm build."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+    if not os.path.exists(HIP_LIB):
+        raise RuntimeError("build the HIP library first (build_hip)")
+    inc = ce.include_paths("cuda") + [sysconfig.get_paths()["include"], INCLUDE]
+    libdirs = ce.library_paths("cuda")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-DTORCH_EXTENSION_NAME=_bf_torch", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-Wno-deprecated-declarations"]
+    cmd += [f"-I{p}" for p in inc]
+    cmd += [os.path.join(CSRC, "bf_torch_ext.cpp"), "-o", TORCH_EXT]
+    cmd += [f"-L{p}" for p in libdirs if os.path.isdir(p)] + [f"-L{HERE}"]
+    cmd += ["-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python", "-lbrokefish_hip",
+            "-Wl,-rpath,$ORIGIN"] + [f"-Wl,-rpath,{p}" for p in libdirs if os.path.isdir(p)]
+    _run(cmd)
+    return TORCH_EXT
+
+
 def build_all(verbose: bool = False) -> None:
     build_chessgen()
     build_hip(verbose)
+    build_torch_ext()

@@ -120,6 +120,29 @@ def load_library():
     return _lib
 
 
+_ext = None
+
+
+def load_extension():
+    """The PyTorch extension module over the same library (``brokefish_amd._bf_torch``: tensors in,
+    launch on the current stream; the counterpart of the reference's extension module,
+    csrc/encoder.cu:1905-1930).  Raises if it has not been built."""
+    global _ext
+    if _ext is None:
+        load_library()
+        try:
+            from . import _bf_torch
+        except ImportError as e:
+            raise RuntimeError(f"the PyTorch extension module is not built ({e}); build it with "
+                               "`python -c 'import __graft_entry__ as g; g.build()'`") from e
+        _ext = _bf_torch
+    return _ext
+
+
+def extension_available() -> bool:
+    return os.path.exists(_build.TORCH_EXT)
+
+
 def int8_q_max():
     """(s8, u8) quantisation maxima compiled into the library."""
     a, b = C.c_double(), C.c_double()
@@ -459,7 +482,14 @@ class FusedEncoder:
     def __init__(self, source, acc_dtype: str = "fp16", fp8: bool = False,
                  int8: Optional[bool] = None, two_boards: Optional[bool] = None,
                  int8_scheme: str = "all", out_dtype: torch.dtype = torch.float16,
-                 device: Optional[torch.device] = None, kernel: str = "auto"):
+                 device: Optional[torch.device] = None, kernel: str = "auto", binding: Optional[str] = None):
+        if binding not in (None, "torch", "ctypes"):
+            raise ValueError(f"binding must be 'torch' (the extension module), 'ctypes' or None, got {binding!r}")
+        # how the launch reaches the library: the PyTorch extension module when it is built (the
+        # default), else the same C-ABI through ctypes; both are one call into libbrokefish_hip.so
+        self.binding = binding or ("torch" if extension_available() else "ctypes")
+        if self.binding == "torch":
+            load_extension()
         if kernel not in self.KERNELS:
             raise ValueError(f"kernel must be one of {tuple(self.KERNELS)}, got {kernel!r}")
         if acc_dtype not in self.ACC_DTYPES:
@@ -734,8 +764,26 @@ class FusedEncoder:
             if active.shape != (n,) or active.dtype not in (torch.uint8, torch.bool) or not active.is_cuda:
                 raise ValueError(f"active must be [{n}] uint8 or bool on the GPU")
             active = active.contiguous().view(torch.uint8)
-        self._call(self._args(boards, control, rep, mask, self.policy_out, self.promo_out,
-                              self.value_out, self.best_out, active=active))
+        if self.binding == "torch":
+            for name, t in (("boards", boards), ("control", control), ("rep", rep), ("mask", mask), ("active", active)):
+                if t is not None and t.device != self.device:
+                    raise ValueError(f"{name} is on {t.device}, the evaluator's weights are on {self.device}")
+            quad = self.wstream is not None
+            if quad:
+                need = self._lib.bf_workspace_bytes(C.byref(self._shape), n)
+                if getattr(self, "workspace", None) is None or self.workspace.numel() < need:
+                    self.workspace = torch.empty(need, device=self.device, dtype=torch.uint8)
+            none = None
+            load_extension().model_forward(
+                boards, control, rep, self.wstream if quad else self.board_wstream,
+                self.fparams if quad else self.board_fparams, self.policy_out, self.promo_out, self.value_out,
+                self.d_model, self.n_layers, self.n_heads, self.d_ff, self.eps, 1 if self.fp8 else 0,
+                self.KERNELS[self.kernel], self.n_value, self.vmode,
+                mask if mask is not None else none, self.best_out if mask is not None else none,
+                active if active is not None else none, self.workspace if quad else none)
+        else:
+            self._call(self._args(boards, control, rep, mask, self.policy_out, self.promo_out,
+                                  self.value_out, self.best_out, active=active))
         self.best_move = self.best_out if mask is not None else None
         return self.policy_out, self.promo_out, self.value_out
 

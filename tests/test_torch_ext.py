@@ -1,0 +1,72 @@
+"""The PyTorch extension module over the C-ABI (brokefish_amd._bf_torch): the counterpart of the
+reference's pybind module (reference csrc/encoder.cu:1770-1876, :1905-1930)."""
+import pytest
+import torch
+
+from brokefish_amd import encoder_impl, hip_impl, positions
+from brokefish_amd.net import BrokefishNet
+
+
+def test_extension_module_loads_and_exports_the_reference_modules_functions():
+    ext = hip_impl.load_extension()
+    for name in ("model_forward", "int8_q_max", "fp8_q_max", "profile_phases", "profile_phase_names", "kernel_choice"):
+        assert hasattr(ext, name), name
+    assert ext.int8_q_max() == (127.0, 255.0) == hip_impl.int8_q_max()
+    assert ext.fp8_q_max() == 8.0
+    assert ext.profile_phase_names()[-1] == "total" and "attention" in ext.profile_phase_names()
+    # AUTO: eight wavefronts per position up to one position per compute unit, the throughput kernel above
+    assert ext.kernel_choice(256, 8, 8, 1024, 1, 64, 0, 0, True) == 4
+    assert ext.kernel_choice(256, 8, 8, 1024, 1, 4096, 0, 0, True) == 3
+    assert ext.kernel_choice(512, 16, 16, 2048, 1, 4096, 0, 0, True) == 4
+    with pytest.raises(RuntimeError):
+        ext.kernel_choice(384, 8, 12, 1536, 1, 64, 0, 0, True)
+    # argument errors are Python RuntimeErrors before any device is touched
+    z = torch.zeros(4, 32, dtype=torch.int16)
+    with pytest.raises(RuntimeError, match="boards must be"):
+        ext.model_forward(z, z, z, z, z, z, z, z, 256, 8, 8, 1024, 1e-5)
+
+
+@pytest.mark.gpu
+def test_extension_binding_returns_the_bits_of_the_ctypes_binding_on_the_current_stream():
+    torch.manual_seed(0)
+    net = BrokefishNet(n_value=3).eval().randomise_layers_(seed=2)
+    b, c, r, m = (t.cuda() for t in positions.random_positions(333, plies=120, seed=9))
+    act = (torch.arange(333, device="cuda") % 3 != 0)
+    for kernel in ("auto", "twin", "octo", "board", "quad"):
+        for fp8 in (False, True):
+            kw = dict(fp8=True) if fp8 else dict(int8=True)
+            te = encoder_impl("hip")(net, kernel=kernel, binding="torch", **kw)
+            ct = encoder_impl("hip")(net, kernel=kernel, binding="ctypes", **kw)
+            assert te.binding == "torch" and ct.binding == "ctypes"
+            want = [t.clone() for t in ct.forward_masked(b, c, r, m)]
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):          # the launch follows torch's current stream
+                got = [t.clone() for t in te.forward_masked(b, c, r, m)]
+            side.synchronize()
+            for g, w in zip(got, want):
+                assert torch.equal(g, w), (kernel, fp8)
+            # the leaf flags reach the kernel through the extension as well
+            for mod in (te, ct):
+                mod.policy_out.fill_(7.0)
+            pa = te.forward_full(b, c, r, active=act)[0].clone()
+            pb = ct.forward_full(b, c, r, active=act)[0].clone()
+            assert torch.equal(pa, pb) and (pa[~act] == 7.0).all()
+    # the default is the extension module when it is built
+    assert encoder_impl("hip")(net, int8=True).binding == "torch"
+    # errors surface as RuntimeError with the library's message
+    ext = hip_impl.load_extension()
+    te = encoder_impl("hip")(net, int8=True, kernel="twin", binding="torch")
+    te.forward_full(b, c, r)
+    bad = torch.empty(10, dtype=torch.uint8, device="cuda")
+    with pytest.raises(RuntimeError, match="not the blobs of this shape"):
+        ext.model_forward(b, c, r, bad, te.board_fparams, te.policy_out, te.promo_out, te.value_out,
+                          256, 8, 8, 1024, 1e-5, n_value=3)
+    with pytest.raises(RuntimeError, match="policy must be"):
+        ext.model_forward(b, c, r, te.board_wstream, te.board_fparams, te.policy_out[:5], te.promo_out[:5], te.value_out[:5],
+                          256, 8, 8, 1024, 1e-5)
+    # the phase profile through the extension
+    cyc = ext.profile_phases(b, c, r, te.board_wstream, te.board_fparams, te.policy_out, te.promo_out, te.value_out,
+                             256, 8, 8, 1024, 1e-5, kernel=3, n_value=3)
+    torch.cuda.synchronize()
+    assert cyc.shape == (12,) and int(cyc[-1]) > 0
