@@ -104,6 +104,8 @@ struct KArgs {
     const uint8_t* rep;
     const uint64_t* mask;
     const uint8_t* active;        // optional [n]: positions with 0 are skipped, their outputs untouched
+    const int* leaf_index;        // optional compacted list: slot j of the launch evaluates position leaf_index[j] ...
+    const int* leaf_count;        // ... for j < *leaf_count; slots past the count do nothing
     int n;
     const uint8_t* wstream;
     const float* fparams;

@@ -259,8 +259,16 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     const int sub = OCTO ? (wave >> 2) : 0;   // which of the quarter's waves it is
     const int t0 = TWW * sub, h0 = HT * sub;  // its first tile of the quarter, its first hidden tile of a step
     const int t = lane & 31, g = lane >> 5;
-    const int b = blockIdx.x;
-    if (a.active && !a.active[b]) return;   // a skipped position: the whole workgroup leaves before any barrier
+    // the position this workgroup evaluates: its own number, or entry blockIdx.x of the compacted
+    // leaf list; a skipped position / a slot past the list's count: the whole workgroup leaves
+    // before any barrier
+    int b = blockIdx.x;
+    if (a.leaf_index) {
+        if (b >= *a.leaf_count) return;
+        b = __builtin_amdgcn_readfirstlane(a.leaf_index[b]);
+        if ((unsigned)b >= (unsigned)a.n) return;   // not a position of this launch
+    }
+    if (a.active && !a.active[b]) return;
     const int nl_run = a.l1 - a.l0;
     // Phase accounting (PROF builds only): the shader clock is read at phase boundaries and the
     // cycles since the previous mark are charged to a slot; the time spent inside workgroup

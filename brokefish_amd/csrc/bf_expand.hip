@@ -38,6 +38,8 @@ struct KExpand {
     const uint16_t* boards;
     const int16_t* control;
     const uint8_t* active;
+    const int* leaf_index;        // optional compacted list: slot j expands position leaf_index[j] for j < *leaf_count
+    const int* leaf_count;
     int n, E, logits_fp32;
     int16_t* edge_move;
     _Float16* edge_prior;
@@ -80,8 +82,13 @@ __device__ __forceinline__ unsigned ordered(float f) {
 
 __global__ __launch_bounds__(256) void expand_kernel(const KExpand a) {
     const int lane = threadIdx.x & 63;
-    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+    int b = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= a.n) return;                       // no workgroup barrier below: a wave may leave
+    if (a.leaf_index) {
+        if (b >= *a.leaf_count) return;
+        b = __builtin_amdgcn_readfirstlane(a.leaf_index[b]);
+        if ((unsigned)b >= (unsigned)a.n) return;   // not a position of this launch
+    }
     if (a.active && !a.active[b]) return;
     const int p = lane >> 1, half = lane & 1;
 
@@ -221,6 +228,51 @@ __global__ __launch_bounds__(256) void expand_kernel(const KExpand a) {
 
 }  // namespace
 
+// Order-preserving compaction of the leaf flags by one workgroup of 1024 lanes: per pass each lane
+// takes one flag; a wave's ballot gives the rank inside the wave, the 16 wave totals are scanned
+// through LDS, and the running total carries over the passes.
+__global__ __launch_bounds__(1024) void compact_kernel(const uint8_t* flags, int n, int* leaf_index, int* leaf_count) {
+    __shared__ int wave_total[16];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int base = 0;
+    for (int lo = 0; lo < n; lo += 1024) {
+        const int i = lo + (int)threadIdx.x;
+        const bool on = i < n && flags[i] != 0;
+        const unsigned long long vote = __ballot(on);
+        const int rank = __builtin_popcountll(vote & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_total[wave] = __builtin_popcountll(vote);
+        __syncthreads();
+        int before = 0, all = 0;
+        for (int w = 0; w < 16; w++) {
+            const int c = wave_total[w];
+            before += w < wave ? c : 0;
+            all += c;
+        }
+        if (on) leaf_index[base + before + rank] = i;
+        base += all;
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *leaf_count = base;
+}
+
+extern "C" int bf_compact_leaves(const uint8_t* flags, int64_t n, int32_t* leaf_index, int32_t* leaf_count, void* stream) {
+    auto fail = [](int code, const char* msg) {
+        bf::set_error(msg);
+        return code;
+    };
+    if (!flags || !leaf_index || !leaf_count) return fail(BF_ERR_ARGUMENT, "flags/leaf_index/leaf_count must not be NULL");
+    if (n < 1 || n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
+    if (((uintptr_t)leaf_index & 3) || ((uintptr_t)leaf_count & 3)) return fail(BF_ERR_ARGUMENT, "leaf_index / leaf_count must be 4-byte aligned");
+    hipLaunchKernelGGL(compact_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, flags, (int)n, leaf_index, leaf_count);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        char msg[256];
+        snprintf(msg, sizeof(msg), "kernel launch failed: %s", hipGetErrorString(e));
+        return fail(BF_ERR_LAUNCH, msg);
+    }
+    return BF_OK;
+}
+
 extern "C" int bf_expand(const bf_expand_args* a, void* stream) {
     auto fail = [](int code, const char* msg) {
         bf::set_error(msg);
@@ -237,7 +289,10 @@ extern "C" int bf_expand(const bf_expand_args* a, void* stream) {
         return fail(BF_ERR_ARGUMENT, "policy must be 16-byte and mask 8-byte aligned");
     KExpand k;
     k.policy = a->policy; k.promo = a->promo; k.value = a->value; k.mask = a->mask;
+    if ((a->leaf_index == nullptr) != (a->leaf_count == nullptr)) return fail(BF_ERR_ARGUMENT, "leaf_index and leaf_count come together");
+    if (a->leaf_index && a->active) return fail(BF_ERR_ARGUMENT, "a compacted leaf list replaces the active flags: pass one of them");
     k.boards = a->boards; k.control = a->control; k.active = a->active;
+    k.leaf_index = a->leaf_index; k.leaf_count = a->leaf_count;
     k.n = (int)a->n; k.E = a->max_edges; k.logits_fp32 = a->logits_fp32 ? 1 : 0;
     k.edge_move = a->edge_move; k.edge_prior = reinterpret_cast<_Float16*>(a->edge_prior);
     k.n_edges = a->n_edges; k.count = a->count; k.dropped = a->dropped;

@@ -151,6 +151,11 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
         ((uintptr_t)a->mask & 7) || ((uintptr_t)a->best_move & 3))
         return fail(BF_ERR_ARGUMENT, "boards/control/value/mask/best_move must be aligned to their element size");
     if (a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
+    if ((a->leaf_index == nullptr) != (a->leaf_count == nullptr))
+        return fail(BF_ERR_ARGUMENT, "leaf_index and leaf_count come together");
+    if (a->leaf_index && a->active) return fail(BF_ERR_ARGUMENT, "a compacted leaf list replaces the active flags: pass one of them");
+    if (((uintptr_t)a->leaf_index & 3) || ((uintptr_t)a->leaf_count & 3))
+        return fail(BF_ERR_ARGUMENT, "leaf_index / leaf_count must be 4-byte aligned");
     if (a->value_mode < BF_VALUE_KING || a->value_mode > BF_VALUE_PRENORM)
         return fail(BF_ERR_ARGUMENT, "value_mode must be BF_VALUE_KING, BF_VALUE_POOLED or BF_VALUE_PRENORM");
     if (a->value_mode != BF_VALUE_KING && !board)
@@ -159,6 +164,7 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
         return fail(BF_ERR_ARGUMENT, "workspace must be 16-byte aligned and hold bf_workspace_bytes(shape, n) bytes");
     memset(k, 0, sizeof(*k));
     k->boards = a->boards; k->control = a->control; k->rep = a->rep; k->mask = a->mask; k->active = a->active;
+    k->leaf_index = a->leaf_index; k->leaf_count = a->leaf_count;
     k->n = (int)a->n;
     k->wstream = ws; k->fparams = fp;
     k->policy = a->policy; k->promo = a->promo; k->value = a->value; k->best = a->best_move;

@@ -143,10 +143,19 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int t = lane & 31, g = lane >> 5;
-    const int board_raw = blockIdx.x * WAVES + wave;
-    // a skipped position keeps its wavefront (the workgroup's barriers need it) but stores nothing
-    const bool valid = board_raw < a.n && !(a.active && !a.active[board_raw < a.n ? board_raw : 0]);
-    const int b = valid ? board_raw : a.n - 1;  // idle waves shadow the last board, store nothing
+    const int board_raw = blockIdx.x * WAVES + wave;   // this wave's slot of the launch (also its workspace slot)
+    // a skipped position keeps its wavefront (the workgroup's barriers need it) but stores nothing;
+    // with a compacted leaf list slot j evaluates position leaf_index[j] while j < *leaf_count
+    bool valid;
+    int b;
+    if (a.leaf_index) {
+        valid = board_raw < a.n && board_raw < *a.leaf_count;
+        b = __builtin_amdgcn_readfirstlane(a.leaf_index[valid ? board_raw : 0]);
+        b = (b >= 0 && b < a.n) ? b : 0;        // an idle wave may read an unwritten entry
+    } else {
+        valid = board_raw < a.n && !(a.active && !a.active[board_raw < a.n ? board_raw : 0]);
+        b = valid ? board_raw : a.n - 1;        // idle waves shadow the last board, store nothing
+    }
 
     Stream st;
     st.t_sync = 0;

@@ -35,8 +35,10 @@ Checked check(const torch::Tensor& boards, const torch::Tensor& control, const t
               const torch::Tensor& promo, const torch::Tensor& value, int64_t d_model, int64_t n_layers,
               int64_t n_heads, int64_t d_ff, double eps, int64_t quant, int64_t kernel, int64_t n_value,
               int64_t vmode, const OptTensor& mask_, const OptTensor& best_move_, const OptTensor& active_,
-              const OptTensor& workspace_) {
+              const OptTensor& workspace_, const OptTensor& leaf_index_ = c10::nullopt,
+              const OptTensor& leaf_count_ = c10::nullopt) {
     const torch::Tensor mask = get(mask_), best_move = get(best_move_), active = get(active_), workspace = get(workspace_);
+    const torch::Tensor leaf_index = get(leaf_index_), leaf_count = get(leaf_count_);
     TORCH_CHECK(boards.is_cuda() && boards.scalar_type() == torch::kShort && boards.is_contiguous() &&
                     boards.dim() == 2 && boards.size(1) == BF_TOKENS,
                 "boards must be [n, 32] int16 contiguous on the GPU");
@@ -66,6 +68,11 @@ Checked check(const torch::Tensor& boards, const torch::Tensor& control, const t
                         active.numel() == n,
                     "active must be [n] uint8 or bool");
     if (!absent(workspace)) TORCH_CHECK(on_dev(workspace) && workspace.scalar_type() == torch::kByte, "workspace must be uint8");
+    TORCH_CHECK(absent(leaf_index) == absent(leaf_count), "leaf_index and leaf_count come together");
+    if (!absent(leaf_index))
+        TORCH_CHECK(on_dev(leaf_index) && on_dev(leaf_count) && leaf_index.scalar_type() == torch::kInt &&
+                        leaf_count.scalar_type() == torch::kInt && leaf_index.numel() >= n && leaf_count.numel() == 1,
+                    "leaf_index must be [n] int32 and leaf_count [1] int32 (see bf_compact_leaves)");
 
     Checked c{bf_eval_args{}, dev};
     bf_eval_args& a = c.a;
@@ -101,6 +108,8 @@ Checked check(const torch::Tensor& boards, const torch::Tensor& control, const t
     a.active = static_cast<const uint8_t*>(ptr_or_null(active));
     a.kernel = (int32_t)kernel;
     a.value_mode = (int32_t)vmode;
+    a.leaf_index = static_cast<const int32_t*>(ptr_or_null(leaf_index));
+    a.leaf_count = static_cast<const int32_t*>(ptr_or_null(leaf_count));
     return c;
 }
 
@@ -108,9 +117,9 @@ void model_forward(torch::Tensor boards, torch::Tensor control, torch::Tensor re
                    torch::Tensor params, torch::Tensor policy, torch::Tensor promo, torch::Tensor value,
                    int64_t d_model, int64_t n_layers, int64_t n_heads, int64_t d_ff, double eps, int64_t quant,
                    int64_t kernel, int64_t n_value, int64_t vmode, OptTensor mask, OptTensor best_move,
-                   OptTensor active, OptTensor workspace) {
+                   OptTensor active, OptTensor workspace, OptTensor leaf_index, OptTensor leaf_count) {
     const Checked c = check(boards, control, rep, weights, params, policy, promo, value, d_model, n_layers, n_heads,
-                            d_ff, eps, quant, kernel, n_value, vmode, mask, best_move, active, workspace);
+                            d_ff, eps, quant, kernel, n_value, vmode, mask, best_move, active, workspace, leaf_index, leaf_count);
     const c10::hip::HIPGuardMasqueradingAsCUDA guard(c.device);     // the launch goes to the tensors' device
     const int rc = bf_model_forward(&c.a, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(c.device.index()).stream());
     TORCH_CHECK(rc == BF_OK, "bf_model_forward failed (", rc, "): ", bf_last_error());
@@ -141,7 +150,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("d_model"), py::arg("n_layers"), py::arg("n_heads"), py::arg("d_ff"), py::arg("eps"),
           py::arg("quant") = 0, py::arg("kernel") = 0, py::arg("n_value") = 1, py::arg("vmode") = 0,
           py::arg("mask") = py::none(), py::arg("best_move") = py::none(), py::arg("active") = py::none(),
-          py::arg("workspace") = py::none());
+          py::arg("workspace") = py::none(), py::arg("leaf_index") = py::none(), py::arg("leaf_count") = py::none());
     m.def("profile_phases", &profile_phases, "cycles per phase of one profiled launch", py::arg("boards"),
           py::arg("control"), py::arg("rep"), py::arg("weights"), py::arg("params"), py::arg("policy"), py::arg("promo"),
           py::arg("value"), py::arg("d_model"), py::arg("n_layers"), py::arg("n_heads"), py::arg("d_ff"), py::arg("eps"),

@@ -56,7 +56,7 @@ class _ExpandArgs(C.Structure):
                 ("boards", C.c_void_p), ("control", C.c_void_p), ("active", C.c_void_p), ("n", C.c_int64),
                 ("max_edges", C.c_int32), ("logits_fp32", C.c_int32), ("edge_move", C.c_void_p),
                 ("edge_prior", C.c_void_p), ("n_edges", C.c_void_p), ("count", C.c_void_p),
-                ("dropped", C.c_void_p), ("node_value", C.c_void_p)]
+                ("dropped", C.c_void_p), ("node_value", C.c_void_p), ("leaf_index", C.c_void_p), ("leaf_count", C.c_void_p)]
 
 
 class _Args(C.Structure):
@@ -67,7 +67,7 @@ class _Args(C.Structure):
                 ("best_move", C.c_void_p), ("out_fp32", C.c_int32), ("quant", C.c_int32),
                 ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("taps", C.POINTER(_Taps)),
                 ("board_wstream", C.c_void_p), ("board_fparams", C.c_void_p), ("active", C.c_void_p),
-                ("kernel", C.c_int32), ("value_mode", C.c_int32)]
+                ("kernel", C.c_int32), ("value_mode", C.c_int32), ("leaf_index", C.c_void_p), ("leaf_count", C.c_void_p)]
 
 
 _lib = None
@@ -111,6 +111,8 @@ def load_library():
         L.bf_expand.argtypes = [C.POINTER(_ExpandArgs), C.c_void_p]
         L.bf_movegen.restype = C.c_int
         L.bf_movegen.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.bf_compact_leaves.restype = C.c_int
+        L.bf_compact_leaves.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p]
         L.bf_board_max_n.restype = C.c_int64
         L.bf_kernel_choice.restype = C.c_int
         L.bf_kernel_choice.argtypes = [C.POINTER(_Args)]
@@ -195,7 +197,39 @@ def movegen(boards, control, out=None):
     return mask, chk
 
 
-def expand_edges(policy, promo, value, mask, boards, control, max_edges: int = 96, active=None, out=None):
+def _check_leaves(leaves, n, device):
+    """(leaf_index [>= n] int32, leaf_count [1] int32) on ``device``, as :func:`compact_leaves` returns them."""
+    index, count = leaves
+    if index.dtype is not torch.int32 or count.dtype is not torch.int32 or index.dim() != 1 or index.shape[0] < n or \
+            count.numel() != 1 or index.device != device or count.device != device or not index.is_contiguous():
+        raise ValueError(f"leaves must be (index [{n}] int32, count [1] int32) on {device}")
+    return index, count
+
+
+def compact_leaves(flags, out=None):
+    """The search's leaf flags ([n] uint8 or bool on the GPU, brokefish/search/cuda_impl.py:137-145)
+    compacted on the device into ``(leaf_index [n] int32, leaf_count [1] int32)``: the numbers of
+    the flagged positions in ascending order and how many there are -- the "compacted list plus a
+    count" of the reference's design retrospective (docs/journal/2026-08-09-kernel-design-
+    retrospective.md:140-154).  ``forward_full(..., leaves=)`` and ``expand_edges(..., leaves=)``
+    take the pair; nothing returns to the host.  ``out`` reuses a pair returned earlier."""
+    if flags.dim() != 1 or flags.dtype not in (torch.uint8, torch.bool) or not flags.is_cuda:
+        raise ValueError("flags must be [n] uint8 or bool on the GPU")
+    n = flags.shape[0]
+    flags = flags.contiguous().view(torch.uint8)
+    if out is None:
+        out = (torch.zeros(n, dtype=torch.int32, device=flags.device), torch.zeros(1, dtype=torch.int32, device=flags.device))
+    index, count = _check_leaves(out, n, flags.device)
+    lib = load_library()
+    with torch.cuda.device(flags.device):
+        rc = lib.bf_compact_leaves(flags.data_ptr(), n, index.data_ptr(), count.data_ptr(),
+                                   C.c_void_p(torch.cuda.current_stream(flags.device).cuda_stream))
+    if rc:
+        raise RuntimeError(f"bf_compact_leaves failed ({rc}): {lib.bf_last_error().decode()}")
+    return index, count
+
+
+def expand_edges(policy, promo, value, mask, boards, control, max_edges: int = 96, active=None, out=None, leaves=None):
     """The search's expand step on the device, behind the evaluator (docs/reference/search.md:616-636,
     brokefish/search/torch_impl.py:962-1033): logits + legal-move words -> edges in canonical order.
 
@@ -204,8 +238,9 @@ def expand_edges(policy, promo, value, mask, boards, control, max_edges: int = 9
     the GPU.  Returns a dict: ``edge_move [n,E]`` int16 (slot*64+square | type << 11), ``edge_prior
     [n,E]`` fp16, ``n_edges [n]`` int32, ``count [n]`` int32 (candidates before truncation to
     ``max_edges``), ``dropped [n]`` fp32 (prior mass truncated away), ``node_value [n]`` fp16 =
-    (value+1)/2.  ``active`` ([n] bool/uint8) leaves the rows where it is 0 untouched; ``out`` reuses
-    a dict returned earlier.  The launch is asynchronous on the current stream."""
+    (value+1)/2.  ``active`` ([n] bool/uint8) leaves the rows where it is 0 untouched, and so does
+    ``leaves`` (the pair :func:`compact_leaves` returns) for positions not in the list; ``out``
+    reuses a dict returned earlier.  The launch is asynchronous on the current stream."""
     n = policy.shape[0]
     if policy.shape != (n, T, N_POLICY) or promo.shape != (n, T, N_PROMO) or policy.dtype != promo.dtype or \
             policy.dtype not in (torch.float16, torch.float32):
@@ -238,6 +273,11 @@ def expand_edges(policy, promo, value, mask, boards, control, max_edges: int = 9
         if act.shape != (n,):
             raise ValueError(f"active must be [{n}]")
         a.active = act.data_ptr()
+    if leaves is not None:
+        if active is not None:
+            raise ValueError("a compacted leaf list replaces the active flags: pass one of them")
+        index, count = _check_leaves(leaves, n, dev)
+        a.leaf_index, a.leaf_count = index.data_ptr(), count.data_ptr()
     a.n, a.max_edges, a.logits_fp32 = n, max_edges, int(policy.dtype is torch.float32)
     a.edge_move, a.edge_prior, a.n_edges = out["edge_move"].data_ptr(), out["edge_prior"].data_ptr(), out["n_edges"].data_ptr()
     a.count, a.dropped, a.node_value = out["count"].data_ptr(), out["dropped"].data_ptr(), out["node_value"].data_ptr()
@@ -646,12 +686,14 @@ class FusedEncoder:
                 raise ValueError(f"{name} must be on the GPU")
         return n
 
-    def _args(self, boards, control, rep, mask, policy, promo, value, best, taps=None, active=None) -> _Args:
+    def _args(self, boards, control, rep, mask, policy, promo, value, best, taps=None, active=None, leaves=None) -> _Args:
         for name, t in (("boards", boards), ("control", control), ("rep", rep), ("mask", mask), ("active", active)):
             if t is not None and t.device != self.device:
                 raise ValueError(f"{name} is on {t.device}, the evaluator's weights are on {self.device}")
         a = _Args()
         a.active = active.data_ptr() if active is not None else None
+        if leaves is not None:
+            a.leaf_index, a.leaf_count = leaves[0].data_ptr(), leaves[1].data_ptr()
         a.boards, a.control, a.rep = boards.data_ptr(), control.data_ptr(), rep.data_ptr()
         a.mask = mask.data_ptr() if mask is not None else None
         a.n = boards.shape[0]
@@ -685,7 +727,7 @@ class FusedEncoder:
             raise RuntimeError(f"bf_kernel_choice failed ({rc}): {self._lib.bf_last_error().decode()}")
         return {1: "quad", 2: "board", 3: "twin", 4: "octo"}[rc]
 
-    def forward_expand(self, boards, control, rep, mask=None, max_edges: int = 96, active=None, out=None):
+    def forward_expand(self, boards, control, rep, mask=None, max_edges: int = 96, active=None, out=None, leaves=None):
         """``forward_full`` followed on the same stream by the search's expand step
         (:func:`expand_edges`), with the legal-move words generated on the device
         (:func:`movegen`) when ``mask`` is not given: two or three launches, no host round trip.
@@ -695,8 +737,8 @@ class FusedEncoder:
         if mask is None:
             mask, chk = movegen(boards, control)
             extra = {"mask": mask, "in_check": chk}
-        policy, promo, value = self.forward_full(boards, control, rep, active=active)
-        edges = expand_edges(policy, promo, value, mask, boards, control, max_edges, active, out)
+        policy, promo, value = self.forward_full(boards, control, rep, active=active, leaves=leaves)
+        edges = expand_edges(policy, promo, value, mask, boards, control, max_edges, active, out, leaves)
         edges.update(extra)
         return edges
 
@@ -746,7 +788,7 @@ class FusedEncoder:
 
     __call__ = forward
 
-    def forward_full(self, boards, control, rep, mask=None, active=None):
+    def forward_full(self, boards, control, rep, mask=None, active=None, leaves=None):
         """Boards to ``(policy_logits, promo, value)`` in one launch.
 
         Without ``mask`` the policy is raw, as the reference evaluator returns it.  With
@@ -754,6 +796,8 @@ class FusedEncoder:
         masked argmax.  Returns views on internal buffers, which the next call overwrites.
         ``active`` ([n] uint8 or bool on the GPU, e.g. the search's leaf flags) skips the
         positions where it is 0: their rows of the output buffers keep what they held.
+        ``leaves`` (the pair :func:`compact_leaves` returns) does the same from a compacted list
+        with a device-side count: only the listed positions are evaluated.
         """
         self._require_net("forward_full")
         n = self._check_inputs(boards, control, rep, mask)
@@ -764,6 +808,10 @@ class FusedEncoder:
             if active.shape != (n,) or active.dtype not in (torch.uint8, torch.bool) or not active.is_cuda:
                 raise ValueError(f"active must be [{n}] uint8 or bool on the GPU")
             active = active.contiguous().view(torch.uint8)
+        if leaves is not None:
+            if active is not None:
+                raise ValueError("a compacted leaf list replaces the active flags: pass one of them")
+            leaves = _check_leaves(leaves, n, self.device)
         if self.binding == "torch":
             for name, t in (("boards", boards), ("control", control), ("rep", rep), ("mask", mask), ("active", active)):
                 if t is not None and t.device != self.device:
@@ -780,10 +828,11 @@ class FusedEncoder:
                 self.d_model, self.n_layers, self.n_heads, self.d_ff, self.eps, 1 if self.fp8 else 0,
                 self.KERNELS[self.kernel], self.n_value, self.vmode,
                 mask if mask is not None else none, self.best_out if mask is not None else none,
-                active if active is not None else none, self.workspace if quad else none)
+                active if active is not None else none, self.workspace if quad else none,
+                leaves[0] if leaves is not None else none, leaves[1] if leaves is not None else none)
         else:
             self._call(self._args(boards, control, rep, mask, self.policy_out, self.promo_out,
-                                  self.value_out, self.best_out, active=active))
+                                  self.value_out, self.best_out, active=active, leaves=leaves))
         self.best_move = self.best_out if mask is not None else None
         return self.policy_out, self.promo_out, self.value_out
 

@@ -172,6 +172,15 @@ typedef struct {
      * (BF_VALUE_PRENORM).  The two pooled heads predict in White's frame and the result is negated
      * when Black is to move (control < 0).  BOARD / TWIN / OCTO kernels; QUAD carries the king head. */
     int32_t value_mode;
+    /* optional compacted leaf list (see bf_compact_leaves): leaf_index [>= *leaf_count] int32 position
+     * numbers and the device-side count.  The launch is sized for n (the size of the flat staging
+     * buffers, an upper bound of the count): workgroup j evaluates position leaf_index[j] and
+     * workgroups past the count leave at once, so no host round trip is needed to learn how many
+     * leaves a simulation step produced.  Inputs are read and outputs written at the position's own
+     * row, as with `active` (which must be NULL when a list is given); rows of positions not in the
+     * list stay untouched.  Both or neither. */
+    const int32_t* leaf_index;
+    const int32_t* leaf_count;
 } bf_eval_args;
 
 /* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */
@@ -280,9 +289,20 @@ typedef struct {
     int32_t* count;
     float* dropped;
     void* node_value;
+    /* optional compacted leaf list, as in bf_eval_args (then `active` must be NULL) */
+    const int32_t* leaf_index;
+    const int32_t* leaf_count;
 } bf_expand_args;
 
 int bf_expand(const bf_expand_args* args, void* stream);
+
+/* Compaction of the search's leaf flags into the list the evaluator and the expansion take: writes
+ * the numbers of the positions whose flag is non-zero, in ascending order, to leaf_index[0 .. count)
+ * and the count to leaf_count[0] (both DEVICE memory; leaf_index holds n entries, entries past the
+ * count are left as they were).  The "compacted list plus a count" of the reference's design
+ * retrospective (reference docs/journal/2026-08-09-kernel-design-retrospective.md:140-154) over its
+ * flat staging (brokefish/search/cuda_impl.py:137-145: leaf_flags).  One workgroup; asynchronous. */
+int bf_compact_leaves(const uint8_t* flags, int64_t n, int32_t* leaf_index, int32_t* leaf_count, void* stream);
 
 /* Legal-move words on the device.  Replaces env.movegen of the reference (reference
  * docs/reference/spec.md:152-172; brokefish/env/torch_impl.py:251-289): for each of n positions

@@ -40,6 +40,7 @@ int main(void) {
     memset(&ex, 0, sizeof ex);
     if (bf_expand(&ex, NULL) != BF_ERR_ARGUMENT || bf_expand(NULL, NULL) != BF_ERR_ARGUMENT) return 12;
     if (bf_movegen(NULL, NULL, 4, NULL, NULL, NULL) != BF_ERR_ARGUMENT) return 13;
+    if (bf_compact_leaves(NULL, 4, NULL, NULL, NULL) != BF_ERR_ARGUMENT) return 17;
     if (bf_mfma_rate(BF_QUANT_INT8, NULL, 10, 1, NULL) >= 0.0) return 14;
     printf("abi ok: %s\n", bf_last_error());
     return 0;

@@ -173,6 +173,51 @@ def test_skipped_positions_keep_their_output_rows(base, kernel):
         model.forward_full(bd, cd, rd, md, active=act[:10])
 
 
+@pytest.mark.parametrize("kernel", ["twin", "octo", "board", "quad"])
+def test_compacted_leaf_list_with_a_device_side_count_equals_the_flag_route(base, kernel):
+    # the "compacted list plus a count" of the reference's design retrospective
+    # (docs/journal/2026-08-09-kernel-design-retrospective.md:140-154) over its flat leaf staging
+    # (brokefish/search/cuda_impl.py:137-145): same rows written, same bits, other rows untouched
+    from brokefish_amd import hip_impl
+    net, sd, boards, quad, co = base
+    model = quad if kernel == "quad" else boards[kernel]
+    b, c, r, m = positions.random_positions(301, plies=120, seed=31)
+    bd, cd, rd, md = _dev(b, c, r, m)
+    g = torch.Generator().manual_seed(4)
+    for flags in (torch.rand(301, generator=g) < 0.4, torch.zeros(301, dtype=torch.bool), torch.ones(301, dtype=torch.bool),
+                  torch.arange(301) == 300):
+        fd = flags.cuda()
+        index, count = hip_impl.compact_leaves(fd)
+        k = int(flags.sum())
+        assert int(count.item()) == k and torch.equal(index[:k].cpu().long(), flags.nonzero()[:, 0])
+        outs = []
+        for route in ("flags", "list"):
+            model.forward_full(bd, cd, rd, md)                      # size the buffers, then mark them
+            for t in (model.policy_out, model.promo_out, model.value_out):
+                t.fill_(7.0)
+            model.best_out.fill_(-7)
+            kw = {"active": fd} if route == "flags" else {"leaves": (index, count)}
+            p, q, v = model.forward_full(bd, cd, rd, md, **kw)
+            outs.append([t.clone() for t in (p, q, v, model.best_out)])
+            assert (v[~fd] == 7.0).all() and (model.best_out[~fd] == -7).all()
+        for x, y in zip(*outs):
+            assert torch.equal(x, y)
+        if k:
+            full = model.forward_full(bd, cd, rd, md)
+            assert torch.equal(outs[1][0][fd], full[0][fd]) and torch.equal(outs[1][2][fd], full[2][fd])
+        # the expansion takes the same list
+        pol, pro, val = [t.clone() for t in model.forward_full(bd, cd, rd)]
+        e1 = {k_: t.clone() for k_, t in hip_impl.expand_edges(pol, pro, val, md, bd, cd, active=fd).items()}
+        e2 = hip_impl.expand_edges(pol, pro, val, md, bd, cd, leaves=(index, count))
+        for k_ in e1:
+            assert torch.equal(e1[k_], e2[k_]), k_
+    with pytest.raises(ValueError):
+        model.forward_full(bd, cd, rd, active=fd, leaves=(index, count))
+    # the chain movegen -> compaction -> evaluator -> expansion stays on the device
+    edges = model.forward_expand(bd, cd, rd, leaves=hip_impl.compact_leaves(torch.arange(301, device="cuda") % 2 == 0))
+    assert (edges["n_edges"][1::2] == 0).all() and (edges["n_edges"][0::2] > 0).any()
+
+
 def test_full_batch_at_4096_on_the_throughput_kernel(base):
     net, sd, boards, quad, co = base
     auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
