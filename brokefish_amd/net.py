@@ -6,7 +6,8 @@ model (brokefish/nn/model.py:276-361): five embedding tables, a pre-norm ReLU
 ``nn.TransformerEncoder`` (deep-copied layers, so a fresh net holds identical layers), a
 final LayerNorm, and three biasless heads; embeddings and heads N(0, 1/sqrt(d)).
 
-The evaluator only *reads* parameters from it (``FusedEncoder(net)`` snapshots them).
+The evaluator only *reads* parameters from it (``FusedEncoder(net)`` snapshots them);
+``forward`` is the plain PyTorch master network a trainer differentiates.
 The three value heads (king row, pooled, prenorm) are carried; re-injection and rule
 features are not (the defaults every published number of the reference uses).
 """
@@ -56,6 +57,50 @@ class BrokefishNet(nn.Module):
         for mod in (self.emb_square, self.emb_type_special, self.emb_color_turn, self.emb_clock,
                     self.emb_rep, self.policy, self.promo, self.value):
             nn.init.normal_(mod.weight, mean=0.0, std=std)
+
+    def forward(self, boards, control, rep, mask=None):
+        """The master network in plain PyTorch, in the parameters' dtype and on their device
+        (reference brokefish/nn/model.py:621-645): ``boards [n,32]`` int16 words, ``control [n]``
+        int16, ``rep [n]`` uint8 -> ``(policy [n,32,64], promo [n,32,4], value [n])``; with ``mask``
+        ([n,32] int64 legal-move words) illegal policy entries are -inf.  This is what a trainer
+        differentiates and what :func:`brokefish_amd.sync.check_weights_propagate` holds a packed
+        evaluator against; the evaluator itself never calls it."""
+        w = boards.to(torch.int64) & 0xFFFF
+        alive = ((w >> 11) & 1) == 0
+        stm = (control < 0).to(torch.int64)
+        i_ts = (((w >> 6) & 7) * 2 + ((w >> 9) & 1)).clamp(max=N_TYPE_SPECIAL - 1)
+        i_ct = ((w >> 10) & 1) * 2 + stm[:, None]
+        i_clock = (control.to(torch.int64).abs() - 1).clamp(0, N_CLOCK - 1)
+        i_rep = rep.to(torch.int64).clamp(0, N_REP - 1)
+        per_board = self.emb_clock(i_clock) + self.emb_rep(i_rep)          # the order of spec 7.2
+        x = self.emb_square(w & 63)
+        x = x + self.emb_type_special(i_ts)
+        x = x + self.emb_color_turn(i_ct)
+        x = x + per_board[:, None, :]
+        h_raw = self.encoder(x, src_key_padding_mask=~alive)
+        h = self.norm_f(h_raw)
+        if self.value_head == "prenorm":
+            m = alive.unsqueeze(-1).to(h_raw.dtype)
+            hv = self.norm_f((h_raw * m).sum(1) / m.sum(1).clamp(min=1))
+        elif self.value_head == "pooled":
+            m = alive.unsqueeze(-1).to(h.dtype)
+            hv = (h * m).sum(1) / m.sum(1).clamp(min=1)
+        else:
+            king = torch.where(control < 0, KING_SLOT_BLACK, KING_SLOT_WHITE).to(torch.int64)
+            hv = h[torch.arange(h.shape[0], device=h.device), king]
+        raw = self.value(hv).float()
+        if self.n_value == 1:
+            value = torch.tanh(raw).squeeze(-1)
+        else:                                   # classes loss, draw, win: p(win) - p(loss)
+            pr = torch.softmax(raw, dim=-1)
+            value = pr[:, 2] - pr[:, 0]
+        if self.value_head != "king":           # the pooled heads predict in White's frame
+            value = torch.where(control > 0, value, -value)
+        policy = self.policy(h)
+        if mask is not None:
+            legal = ((mask.to(torch.int64)[..., None] >> torch.arange(64, device=mask.device)) & 1).bool()
+            policy = policy.masked_fill(~legal, float("-inf"))
+        return policy, self.promo(h), value
 
     @torch.no_grad()
     def randomise_layers_(self, seed: int = 1, scale: float = 1.0) -> "BrokefishNet":

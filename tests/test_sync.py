@@ -5,6 +5,7 @@
 formula-weight network (tests/golden/make_golden.py) and by its defining properties: it moves
 when a value moves and when two values swap places.
 """
+import numpy as np
 import pytest
 import torch
 
@@ -102,3 +103,61 @@ def test_checkpoint_conventions_size_a_net_from_a_bare_state_dict():
         bn.value_head_of(dict(state, value_mode=torch.tensor(9)))
     with pytest.raises(ValueError):
         bn.rule_features_of(dict(state, rule_features_mode=torch.tensor(2)))
+
+
+def test_master_network_forward_is_the_fp32_restatement_and_the_references_golden(golden):
+    # brokefish_amd.net.BrokefishNet.forward against the checker's fp32 route and against the logits
+    # the reference's own model wrote for the formula weights (brokefish/nn/model.py:621-645)
+    import make_golden as mg
+    from oracle import emulated
+    for head, nv in (("king", 1), ("king", 3), ("pooled", 3), ("prenorm", 1)):
+        torch.manual_seed(0)
+        net = BrokefishNet(n_value=nv, value_head=head).eval()
+        net.load_state_dict(mg.fill_state_dict(net.state_dict()))
+        b, c, r = mg.positions()
+        with torch.no_grad():
+            got = net(b, c, r)
+            want = emulated.forward({k: v for k, v in net.state_dict().items()}, b, c, r, mode="fp32")
+        for g, w in zip(got, want):
+            assert (g - w).abs().max() < 2e-5
+        if head == "king":
+            nb = 3 if nv == 3 else 8
+            assert np.abs(got[0].numpy()[:nb] - golden[f"fp32_policy_nv{nv}"]).max() < 2e-5
+            assert np.abs(got[2].numpy()[:nb] - golden[f"fp32_value_nv{nv}"]).max() < 2e-6
+    m = torch.full((8, 32), 0x0F0F, dtype=torch.int64)
+    with torch.no_grad():
+        pm = net(b, c, r, mask=m)[0]
+    assert torch.isneginf(pm[:, :, 4]).all() and torch.isfinite(pm[:, :, 0]).all()
+
+
+@pytest.mark.gpu
+def test_start_up_consistency_check_catches_a_stale_snapshot_a_nan_and_a_wrong_slab():
+    # reference brokefish/train/loop.py:1109-1166 (check 9 of its training loop)
+    for kw in ({"int8": True}, {"fp8": True}):
+        torch.manual_seed(0)
+        net = BrokefishNet().eval()
+        packed = sync.PackedWeights.pack(net, 0, **kw)
+        fp_before = sync.weight_fingerprint(net)
+        res = sync.check_weights_propagate(net, packed)
+        assert res["moved"] > 0 and res["agree"] <= res["tol"] and sync.weight_fingerprint(net) == fp_before
+    # a stale snapshot: packing hands back the evaluator of the old weights
+    real_pack = sync.PackedWeights.pack
+    try:
+        sync.PackedWeights.pack = classmethod(lambda cls, *a, **k: packed)
+        with pytest.raises(AssertionError, match="did not change"):
+            sync.check_weights_propagate(net, packed)
+        # a wrong weight slab: the repacked evaluator holds another network's weights
+        torch.manual_seed(7)
+        other = real_pack(BrokefishNet().eval().randomise_layers_(seed=8, scale=3.0), 1, int8=True)
+        sync.PackedWeights.pack = classmethod(lambda cls, *a, **k: other)
+        with pytest.raises(AssertionError, match="disagrees"):
+            sync.check_weights_propagate(net, packed)
+    finally:
+        sync.PackedWeights.pack = real_pack
+    # a non-finite output is an error, not a pass (nan > tol is False)
+    torch.manual_seed(0)
+    bad = BrokefishNet().eval()
+    with torch.no_grad():
+        bad.norm_f.weight[3] = float("nan")
+    with pytest.raises(AssertionError, match="non-finite"):
+        sync.check_weights_propagate(bad, sync.PackedWeights.pack(bad, 0, int8=True))
