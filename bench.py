@@ -60,6 +60,35 @@ def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0, mode: st
                       f"os.cpu_count()={os.cpu_count()}"}
 
 
+def physical_cores() -> int:
+    """Physical cores this process may run on: distinct (package, core) pairs of /proc/cpuinfo among the
+    CPUs of the affinity mask (hardware threads of one core count once)."""
+    try:
+        allowed = os.sched_getaffinity(0)
+        seen, cpu, phys = set(), None, 0
+        for line in open("/proc/cpuinfo"):
+            k, _, v = line.partition(":")
+            k, v = k.strip(), v.strip()
+            if k == "processor":
+                cpu = int(v)
+            elif k == "physical id":
+                phys = int(v)
+            elif k == "core id" and cpu in allowed:
+                seen.add((phys, int(v)))
+        return len(seen) or len(allowed)
+    except OSError:
+        return os.cpu_count() or 1
+
+
+def time_config(net, fmt, batch, kernel="auto", iters=20, warmup=3):
+    """(kernel ms per launch from HIP events on the launch stream, kernel name) for one configuration."""
+    from brokefish_amd import encoder_impl, positions
+    model = encoder_impl("hip")(net, fp8=True, kernel=kernel) if fmt == "e4m3" else encoder_impl("hip")(net, int8=True, kernel=kernel)
+    sb, sc, sr, sm = (t.cuda() for t in positions.random_positions(batch, plies=120, seed=0))
+    ms = model.time_kernel_ms(sb, sc, sr, sm, warmup=warmup, iters=iters)
+    return ms, model.kernel_choice(batch), model
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -75,8 +104,9 @@ def main() -> int:
                     help="four positions per workgroup; one position per workgroup with one (board; octo: eight wavefronts) or two (twin) workgroups per compute unit; auto: by batch size")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=64)
-    ap.add_argument("--sweep", action="store_true",
-                    help="also time batch sizes 64..65536 (per-launch latency regime) and add them to the line")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="headline only: skip the batch sweep, the e4m3 and stress configurations and the parity report")
+    ap.add_argument("--sweep", action="store_true", help="(kept for older command lines: the sweep is part of the default line)")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one device copy of this many MiB (a kernel of known HBM traffic, "
                          "to calibrate FETCH_SIZE / WRITE_SIZE counter runs)")
@@ -91,6 +121,7 @@ def main() -> int:
     from brokefish_amd.net import BrokefishNet
 
     stress = a.shape == "stress"
+    headline = not stress and a.quant == "int8" and a.batch in (None, 4096)
     if a.batch is None:
         a.batch = 16384 if stress else 4096
     ops_per_eval = OPS_PER_EVAL_STRESS if stress else OPS_PER_EVAL
@@ -123,6 +154,9 @@ def main() -> int:
     kern_ms = model.time_kernel_ms(bd, cd, rd, md, warmup=3, iters=max(a.steps, 10))
     achieved = ops_per_eval * a.batch / (kern_ms * 1e-3) / 1e12
     peak = PEAK_FP16_OPS if fp8 else PEAK_INT8_OPS
+    kname = model.kernel_choice(a.batch)
+    traffic = (MEASURED_TRAFFIC_BYTES_E4M3 if fp8 else MEASURED_TRAFFIC_BYTES).get((a.shape, kname, a.batch))
+    weight_bytes = (50_626_560 if stress else 6_455_296) * a.batch      # each position streams its own copy from L2
     line = {
         "metric": (f"network evals/sec at batch {a.batch} int8, 16-layer width-512 stress shape, on 1 MI355X" if stress
                    else f"network evals/sec at batch 4096 {'fp8 e4m3' if fp8 else 'int8'} on 1 MI355X"),
@@ -131,34 +165,85 @@ def main() -> int:
         "dtype": "fp8" if fp8 else "int8", "data": "synthetic",
         "config": {"workload": (f"configs[4]: 16-layer d512 16-head FFN2048 int8 evaluator, batch {a.batch}, " if stress else
                                 f"configs[{3 if fp8 else 1}]: 8-layer d256 8-head FFN1024 {a.quant} evaluator, batch {a.batch}, ")
-                               + f"kernel {model.kernel_choice(a.batch)}, "
+                               + f"kernel {kname}, binding {model.binding}, "
                                "seeded random playouts 0-120 plies, legal-move mask ANDed in-kernel, "
                                "fp16 logits out, seed-0 random-init weights"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": peak / 1e12, "unit": "TFLOP/s" if fp8 else "TOP/s",
                      "frac": achieved / (peak / 1e12),
-                     "traffic": (MEASURED_TRAFFIC_BYTES_E4M3 if fp8 else MEASURED_TRAFFIC_BYTES).get(
-                         (a.shape, model.kernel_choice(a.batch), a.batch)),
-                     "kernel_ms": kern_ms, "ops_per_launch": ops_per_eval * a.batch},
+                     # HBM bytes per launch: not measurable inside this process; the figure is the
+                     # FETCH_SIZE + WRITE_SIZE counter result of the same command summarised under profiles/
+                     "traffic": traffic, "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (not measured in this run)" if traffic else None,
+                     "kernel_ms": kern_ms, "ops_per_launch": ops_per_eval * a.batch,
+                     # what bounds the kernel in practice: every position streams the packed weights from
+                     # L2 through its compute unit's vector L1, whose fill path moves 64 bytes per clock
+                     "weight_stream": {"bytes_per_launch": weight_bytes, "achieved_TBps": weight_bytes / (kern_ms * 1e-3) / 1e12,
+                                       "l1_fill_peak_TBps": 256 * 64 * 2.4e9 / 1e12}},
     }
     # the matrix pipe's measured ceiling for the instruction the kernel uses (register-resident
     # MFMA chains, no memory traffic), next to the datasheet peak that `frac` is quoted against
     from brokefish_amd.hip_impl import mfma_rate
     line["roofline"]["measured_mfma_rate"] = mfma_rate(a.quant)
-    if a.sweep:
-        # the batch-size sweep of the small-batch latency regime: same net, same generator
+    del model, bd, cd, rd, md
+    if headline and not a.no_extras:
+        # configuration 3: the batch sweep (small-batch latency regime), same net, same generator
         pts = []
         for nb in (64, 256, 1024, 4096, 16384, 65536):
-            sb, sc, sr, sm = (t.cuda() for t in positions.random_positions(nb, plies=120, seed=0))
-            ms = model.time_kernel_ms(sb, sc, sr, sm, warmup=3, iters=20)
-            pts.append({"batch": nb, "ms_per_launch": ms, "evals_per_s": nb / ms * 1e3,
-                        "kernel": model.kernel_choice(nb)})
-            del sb, sc, sr, sm
+            ms, kn, mdl = time_config(net, "int8", nb, iters=20 if nb <= 16384 else 8)
+            pts.append({"batch": nb, "ms_per_launch": ms, "evals_per_s": nb / ms * 1e3, "kernel": kn,
+                        "frac_int8_peak": OPS_PER_EVAL * nb / (ms * 1e-3) / PEAK_INT8_OPS})
+            del mdl
         line["sweep"] = pts
+        # configuration 4: e4m3 at batch 4096 (products on the fp16 matrix instruction: quoted against both peaks)
+        ms, kn, mdl = time_config(net, "e4m3", 4096)
+        tops = OPS_PER_EVAL * 4096 / (ms * 1e-3)
+        line["e4m3"] = {"batch": 4096, "kernel": kn, "kernel_ms": ms, "evals_per_s": 4096 / ms * 1e3, "achieved_TFLOPs": tops / 1e12,
+                        "frac_fp16_peak_2.5PF": tops / PEAK_FP16_OPS, "frac_fp8_peak_5.0PF": tops / 5.0e15,
+                        "measured_mfma_rate": mfma_rate("e4m3")}
+        del mdl
+        # configuration 5: the 16-layer 512-wide network at batch 16384
+        torch.manual_seed(0)
+        wide = BrokefishNet(d_model=512, n_heads=16, d_ff=2048, n_layers=16).eval()
+        ms, kn, mdl = time_config(wide, "int8", 16384, iters=5, warmup=2)
+        line["stress"] = {"batch": 16384, "kernel": kn, "kernel_ms": ms, "evals_per_s": 16384 / ms * 1e3,
+                          "achieved_TOPs": OPS_PER_EVAL_STRESS * 16384 / (ms * 1e-3) / 1e12,
+                          "frac_int8_peak": OPS_PER_EVAL_STRESS * 16384 / (ms * 1e-3) / PEAK_INT8_OPS}
+        del mdl, wide
+        line["parity"] = parity_report(net)
     if not a.no_cpu:
-        threads = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
-        line["cpu_baseline"] = cpu_baseline(net, a.cpu_batch, threads, mode=a.quant)
+        cores = physical_cores()
+        threads = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+        line["cpu_baseline"] = cpu_baseline(net, a.cpu_batch, threads, mode=a.quant, budget_s=12.0)
+        line["cpu_baseline"]["physical_cores"] = cores
+        if headline and not a.no_extras:      # configuration 1 names fp32 and the int8 simulation
+            f32 = cpu_baseline(net, a.cpu_batch, threads, mode="fp32", budget_s=4.0)
+            line["cpu_baseline"]["fp32"] = {"value": f32["value"], "unit": "evals/s", "sample": f32["sample"]}
     print(json.dumps(line))
     return 0
+
+
+def parity_report(net):
+    """What is checked next to the number: a sample of the batch bit for bit against the C checker,
+    and the prior-space distance to the int8 emulation as the reference reports it
+    (brokefish/nn/validate.py:314-388: max |dp|, 95th percentile, top-1 moved, flip)."""
+    import numpy as np
+    import torch
+    from brokefish_amd import encoder_impl, positions, validate
+    from oracle import c_oracle, emulated
+    sd = {k: v.detach() for k, v in net.state_dict().items()}
+    b, c, r, m = positions.random_positions(128, plies=120, seed=1)
+    bd, cd, rd, md = b.cuda(), c.cuda(), r.cuda(), m.cuda()
+    model = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
+    got = [t.clone() for t in model.forward_masked(bd, cd, rd, md)]
+    want = c_oracle.COracle(sd).forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy())
+    exact = all((g.cpu().numpy().view(np.int32) == want[k].view(np.int32)).all()
+                for k, g in (("policy", got[0]), ("promo", got[1]), ("value", got[2]))) and \
+        bool((got[3].cpu().numpy() == want["best"]).all())
+    with torch.no_grad():
+        emu = emulated.forward(sd, b, c, r, mode="int8")
+    raw = [t.clone() for t in model.forward_full(bd, cd, rd)]
+    d = validate.compare("kernel vs int8 emulation", tuple(t.cuda() for t in emu), raw, md, bd, cd)
+    return {"positions": 128, "bit_exact_vs_c_checker": bool(exact), "masked_argmax_equal": bool((got[3].cpu().numpy() == want["best"]).all()),
+            "prior_space_vs_int8_emulation": {k: v for k, v in d.as_dict().items() if k != "name"}}
 
 
 if __name__ == "__main__":

@@ -19,7 +19,7 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 @pytest.mark.gpu
 def test_one_json_line_with_roofline_and_cpu_baseline():
     run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "5", "--warmup", "2", "--cpu-batch", "16"],
-                         capture_output=True, text=True, timeout=280)
+                         capture_output=True, text=True, timeout=400)
     assert run.returncode == 0, run.stderr[-2000:]
     lines = [l for l in run.stdout.splitlines() if l.strip()]
     assert len(lines) == 1
@@ -38,3 +38,15 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert d["value"] > 1.0e6          # a sanity bound, far below what the kernel measures (2.1-2.2 M)
     c = d["cpu_baseline"]
     assert c["kind"] == "port" and c["unit"] == "evals/s" and c["cores"] >= 1 and c["value"] > 0 and "batch 16" in c["sample"]
+    assert c["physical_cores"] >= 1 and c["fp32"]["value"] > 0
+    # every configuration is in the default line: the sweep, e4m3 and the 512-wide network
+    assert [p["batch"] for p in d["sweep"]] == [64, 256, 1024, 4096, 16384, 65536]
+    assert all(p["ms_per_launch"] > 0 and p["kernel"] in ("octo", "twin") for p in d["sweep"])
+    e = d["e4m3"]
+    assert e["batch"] == 4096 and abs(e["frac_fp16_peak_2.5PF"] - 2 * e["frac_fp8_peak_5.0PF"]) < 1e-9 and e["evals_per_s"] > 5e5
+    st = d["stress"]
+    assert st["batch"] == 16384 and st["kernel"] == "octo" and 0.05 < st["frac_int8_peak"] < 1.0
+    par = d["parity"]
+    assert par["bit_exact_vs_c_checker"] is True and par["masked_argmax_equal"] is True
+    assert par["prior_space_vs_int8_emulation"]["max_abs"] < 1e-2 and par["prior_space_vs_int8_emulation"]["edge_set_differs"] == 0
+    assert r["weight_stream"]["bytes_per_launch"] == 4096 * 6_455_296
