@@ -431,7 +431,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
                 for (int u = 0; u < SUB; u++) m = __builtin_fmaxf(m, xch[2 * XS + (w + 4 * u) * 64 + lane]);
             m = __builtin_fmaxf(m, partner(m, g));
-            sa[c] = m > 0.0f ? m / (FP8 ? 8.0f : 127.0f) : 1.0f;
+            sa[c] = m > 0.0f ? (FP8 ? m * 0.125f : div127(m)) : 1.0f;
         }
         const float so = KC == 1 ? sa[0] : (q < WPC ? sa[0] : sa[KC - 1]);
         const float inv = 1.0f / so;
@@ -803,7 +803,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                         m = __builtin_fmaxf(m, __builtin_fmaxf(xch[xs + (2 * c + 4 * u) * 64 + lane],
                                                                xch[xs + (2 * c + 1 + 4 * u) * 64 + lane]));
                     m = __builtin_fmaxf(m, partner(m, g));
-                    sh[2 * st + c] = m > 0.0f ? m / (FP8 ? 8.0f : 255.0f) : 1.0f;
+                    sh[2 * st + c] = m > 0.0f ? (FP8 ? m * 0.125f : div255(m)) : 1.0f;
                 }
                 const float s8 = q < 2 ? sh[2 * st] : sh[2 * st + 1];
                 const float inv = 1.0f / s8;
@@ -955,7 +955,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                             m = __builtin_fmaxf(m, __builtin_fmaxf(xch[2 * XS + (2 * c + 4 * u) * 64 + lane],
                                                                    xch[2 * XS + (2 * c + 1 + 4 * u) * 64 + lane]));
                         m = __builtin_fmaxf(m, partner(m, g));
-                        sh[c] = m > 0.0f ? m / (FP8 ? 8.0f : 255.0f) : 1.0f;
+                        sh[c] = m > 0.0f ? (FP8 ? m * 0.125f : div255(m)) : 1.0f;
                     }
                     const float s8 = q < 2 ? sh[0] : sh[1];
                     const float inv = 1.0f / s8;

@@ -137,6 +137,20 @@ __device__ __forceinline__ float accf(const v16f& a, int i) { return a[i]; }
 __device__ __forceinline__ int accbits(const v16i& a, int i) { return a[i]; }
 __device__ __forceinline__ int accbits(const v16f& a, int i) { return __float_as_int(a[i]); }
 
+// m / 127 and m / 255 (the activation scales), correctly rounded for every finite m: the
+// reciprocal constant and two fused corrections.  Equal to IEEE division on all 2^31 positive
+// floats, subnormals included (checked exhaustively on the CPU), and a third of its instructions.
+__device__ __forceinline__ float div127(float m) {
+    const float c = 1.0f / 127.0f;
+    const float q = m * c;
+    return __builtin_fmaf(__builtin_fmaf(-q, 127.0f, m), c, q);
+}
+__device__ __forceinline__ float div255(float m) {
+    const float c = 1.0f / 255.0f;
+    const float q = m * c;
+    return __builtin_fmaf(__builtin_fmaf(-q, 255.0f, m), c, q);
+}
+
 // ---- row operations -------------------------------------------------------------------
 
 // four quotients v / sa (correctly rounded) -> one packed dword.
@@ -160,14 +174,16 @@ __device__ __forceinline__ unsigned quant4(float v0, float v1, float v2, float v
         w = __builtin_amdgcn_cvt_pk_fp8_f32(qf[2], qf[3], w, true);
         return (unsigned)w;
     } else {
-        unsigned m[4];
-        // adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low bits
-#pragma unroll
-        for (int i = 0; i < 4; i++) m[i] = (unsigned)__float_as_int(qf[i] + 12582912.0f);
-        // gather the four low bytes with byte permutes (selector 0-3: second operand, 4-7: first, 0x0c: zero)
-        const unsigned lo = __builtin_amdgcn_perm(m[1], m[0], 0x0c0c0400u);
-        const unsigned hi = __builtin_amdgcn_perm(m[3], m[2], 0x04000c0cu);
-        return lo | hi;
+        // Adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low bits of the sum;
+        // the sub-dword form of the add writes that low byte straight into its place in the packed
+        // dword (checked on the GPU against rint on four million values and the ties).
+        const float magic = 12582912.0f;
+        unsigned w;
+        asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(w) : "v"(qf[0]), "v"(magic));
+        asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(w) : "v"(qf[1]), "v"(magic));
+        asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(w) : "v"(qf[2]), "v"(magic));
+        asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(w) : "v"(qf[3]), "v"(magic));
+        return w;
     }
 }
 
@@ -198,7 +214,7 @@ __device__ __forceinline__ void quant_s8(const float (&y)[NTILES][16], int g, v4
 #pragma unroll
         for (int r = 0; r < 16; r++) am = __builtin_fmaxf(am, __builtin_fabsf(y[n][r]));
     am = __builtin_fmaxf(am, partner(am, g));
-    sa = am > 0.0f ? am / (FP8 ? 8.0f : 127.0f) : 1.0f;
+    sa = am > 0.0f ? (FP8 ? am * 0.125f : div127(am)) : 1.0f;
     const float inv = 1.0f / sa;
 #pragma unroll
     for (int n = 0; n < NTILES; n++)

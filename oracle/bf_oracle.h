@@ -50,6 +50,7 @@ typedef struct {
 
 typedef struct bfo_model bfo_model;
 
+long bfo_check_div_const(float D, unsigned stride);
 float bfo_exp_neg(float x);
 float bfo_tanh(float x);
 void bfo_quantise_weights_int8(const float* w, int n, int k, int8_t* q, float* scale);

@@ -66,6 +66,8 @@ def lib():
         L.bfo_forward.argtypes = [C.c_void_p] + [C.c_void_p] * 4 + [C.c_int] + [C.c_void_p] * 4 + [C.POINTER(_Taps)]
         L.bfo_exp_neg.restype = C.c_float
         L.bfo_exp_neg.argtypes = [C.c_float]
+        L.bfo_check_div_const.restype = C.c_long
+        L.bfo_check_div_const.argtypes = [C.c_float, C.c_uint]
         L.bfo_tanh.restype = C.c_float
         L.bfo_tanh.argtypes = [C.c_float]
         L.bfo_quantise_weights_int8.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
