@@ -142,7 +142,10 @@ def load_extension():
 
 
 def extension_available() -> bool:
-    return os.path.exists(_build.TORCH_EXT)
+    """Whether the default binding is the extension module.  The module is linked against the
+    in-tree library, so a ``BROKEFISH_HIP_LIB`` override (another build of the library) selects
+    the ctypes binding, which loads the named file."""
+    return os.path.exists(_build.TORCH_EXT) and "BROKEFISH_HIP_LIB" not in os.environ
 
 
 def int8_q_max():

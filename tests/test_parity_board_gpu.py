@@ -67,6 +67,26 @@ def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base, kerne
 
 
 @pytest.mark.parametrize("kernel", ["board", "twin", "octo"])
+def test_heads_alone_and_a_layer_range_from_a_given_residual_stream(base, kernel):
+    # a run of no layers starts the weight stream at the head blocks (no layer block is fetched,
+    # none exists to fetch past the last layer); a run of some layers continues into them
+    net, sd, boards, quad, co = base
+    model = boards[kernel]
+    b, c, r, m = positions.random_positions(37, plies=90, seed=29)
+    bd, cd, rd, md = _dev(b, c, r, m)
+    want = co.forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy(), taps=True)
+    heads = model.forward_taps(bd, cd, rd, mask=md, x_in=torch.from_numpy(want["resid"][:, 7]).cuda(),
+                               layer_begin=8, layer_end=8, want=["normed"])
+    for k in ("normed", "policy", "promo", "value", "best"):
+        assert _bits_equal(heads[k], want[k]), k
+    tail = model.forward_taps(bd, cd, rd, mask=md, x_in=torch.from_numpy(want["resid"][:, 4]).cuda(),
+                              layer_begin=5, layer_end=8, want=["resid"])
+    assert _bits_equal(tail["resid"][:, -1], want["resid"][:, 7])
+    for k in ("policy", "promo", "value", "best"):
+        assert _bits_equal(tail[k], want[k]), k
+
+
+@pytest.mark.parametrize("kernel", ["board", "twin", "octo"])
 @pytest.mark.parametrize("nv", [1, 3])
 def test_the_kernels_return_the_same_bits(base, nv, kernel):
     if nv == 1:
