@@ -174,11 +174,17 @@ def main() -> int:
                      # FETCH_SIZE + WRITE_SIZE counter result of the same command summarised under profiles/
                      "traffic": traffic, "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (not measured in this run)" if traffic else None,
                      "kernel_ms": kern_ms, "ops_per_launch": ops_per_eval * a.batch,
-                     # what bounds the kernel in practice: every position streams the packed weights from
-                     # L2 through its compute unit's vector L1, whose fill path moves 64 bytes per clock
+                     # the kernel's second resource: every position streams the packed weights out of the
+                     # cache hierarchy (bytes_per_launch / kernel_ms = achieved); `stream_ceiling_TBps` is
+                     # what the same number of workgroups reach streaming a buffer of the network's size
+                     # with nothing else to do (measured below), `l1_fill_nominal_TBps` 64 bytes per clock
+                     # and compute unit
                      "weight_stream": {"bytes_per_launch": weight_bytes, "achieved_TBps": weight_bytes / (kern_ms * 1e-3) / 1e12,
-                                       "l1_fill_peak_TBps": 256 * 64 * 2.4e9 / 1e12}},
+                                       "l1_fill_nominal_TBps": 256 * 64 * 2.4e9 / 1e12}},
     }
+    from brokefish_amd.hip_impl import stream_rate
+    line["roofline"]["weight_stream"]["stream_ceiling_TBps"] = stream_rate(weight_bytes // a.batch, workgroups=min(a.batch, 4096),
+                                                                           reps=1 if stress else 3)
     # the matrix pipe's measured ceiling for the instruction the kernel uses (register-resident
     # MFMA chains, no memory traffic), next to the datasheet peak that `frac` is quoted against
     from brokefish_amd.hip_impl import mfma_rate

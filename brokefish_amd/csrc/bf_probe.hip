@@ -70,6 +70,31 @@ __global__ __launch_bounds__(PROBE_THREADS) void mfma_loop(int* scratch, int ite
     if (fold == 0x5bd1e995) scratch[512 + lane] = fold;
 }
 
+// Weight-stream probe: every workgroup reads the whole buffer once, as a position's workgroup
+// reads the whole network -- wavefront w its quarter, 16 bytes per lane and load, eight loads in
+// flight, nothing else in the loop.  Workgroups start at different offsets of their quarters
+// (they are at different layers in the evaluator too) and wrap around.
+constexpr int STREAM_AHEAD = 8;
+__global__ __launch_bounds__(PROBE_THREADS) void stream_loop(const uint8_t* buf, size_t chunks_per_quarter, int* sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint8_t* base = buf + (size_t)wave * chunks_per_quarter * 1024 + lane * 16;
+    const size_t start = ((size_t)blockIdx.x * 2654435761u) % chunks_per_quarter;
+    v4i acc = {0, 0, 0, 0};
+    for (size_t c = 0; c < chunks_per_quarter; c += STREAM_AHEAD) {
+        v4i v[STREAM_AHEAD];
+#pragma unroll
+        for (int u = 0; u < STREAM_AHEAD; u++) {
+            size_t idx = start + c + u;
+            if (idx >= chunks_per_quarter) idx -= chunks_per_quarter;
+            v[u] = *reinterpret_cast<const v4i*>(base + idx * 1024);
+        }
+#pragma unroll
+        for (int u = 0; u < STREAM_AHEAD; u++) acc ^= v[u];
+    }
+    // keeps the loads alive; never true for a buffer of equal 32-bit words (the xor of an even count is 0)
+    if ((acc[0] ^ acc[1]) == 0x5bd1e995 && (acc[2] ^ acc[3]) == 0x1b873593) sink[lane] = acc[0];
+}
+
 }  // namespace
 
 extern "C" double bf_mfma_rate(int quant, int* scratch, int iters, int reps, void* stream) {
@@ -109,4 +134,35 @@ extern "C" double bf_mfma_rate(int quant, int* scratch, int iters, int reps, voi
     // 2*32*32*32 operations per int8 instruction; the e4m3 chain step is two 32x32x16 fp16 instructions
     const double ops = 65536.0 * CHAINS * (double)iters * (PROBE_THREADS / 64) * grid.x * reps;
     return ops / ((double)ms * 1e-3) / 1e12;
+}
+
+extern "C" double bf_stream_rate(const void* buf, size_t bytes, int workgroups, int reps, int* sink, void* stream) {
+    auto fail = [](int code, const char* msg) {
+        bf::set_error(msg);
+        return (double)code;
+    };
+    constexpr size_t UNIT = (size_t)4 * STREAM_AHEAD * 1024;   // four quarters of whole groups of loads
+    if (!buf || ((uintptr_t)buf & 15) || !sink) return fail(BF_ERR_ARGUMENT, "buf must be a 16-byte aligned device buffer and sink 256 device bytes");
+    if (bytes < UNIT || bytes % UNIT) return fail(BF_ERR_ARGUMENT, "bytes must be a positive multiple of 32768");
+    if (workgroups < 1 || workgroups > (1 << 20) || reps < 1 || reps > 1000) return fail(BF_ERR_ARGUMENT, "workgroups must be in [1, 2^20] and reps in [1, 1000]");
+    hipStream_t s = (hipStream_t)stream;
+    auto go = [&]() { hipLaunchKernelGGL(stream_loop, dim3(workgroups), dim3(PROBE_THREADS), 0, s, (const uint8_t*)buf, bytes / 4096, sink); };
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess) return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    if (hipEventCreate(&e1) != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return fail(BF_ERR_LAUNCH, "hipEventCreate failed");
+    }
+    go();                                               // warm-up: the buffer into the caches
+    (void)hipEventRecord(e0, s);
+    for (int r = 0; r < reps; r++) go();
+    (void)hipEventRecord(e1, s);
+    const hipError_t e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    (void)hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    const hipError_t le = hipGetLastError();
+    if (e != hipSuccess || le != hipSuccess) return fail(BF_ERR_LAUNCH, hipGetErrorString(e != hipSuccess ? e : le));
+    return (double)bytes * workgroups * reps / ((double)ms * 1e-3) / 1e12;
 }

@@ -118,6 +118,8 @@ def load_library():
         L.bf_kernel_choice.argtypes = [C.POINTER(_Args)]
         L.bf_mfma_rate.restype = C.c_double
         L.bf_mfma_rate.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
+        L.bf_stream_rate.restype = C.c_double
+        L.bf_stream_rate.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
         _lib = L
     return _lib
 
@@ -171,6 +173,23 @@ def mfma_rate(fmt: str = "int8", iters: int = 20000, reps: int = 5, device="cuda
                               torch.cuda.current_stream().cuda_stream)
     if rate < 0:
         raise RuntimeError(f"bf_mfma_rate: {L.bf_last_error().decode()}")
+    return float(rate)
+
+
+def stream_rate(nbytes: int, workgroups: int = 4096, reps: int = 3, device="cuda") -> float:
+    """Measured rate in TB/s at which ``workgroups`` workgroups can each stream the same ``nbytes``
+    (rounded up to a multiple of 32 KiB) out of the cache hierarchy with nothing else to do: the
+    ceiling for the evaluator's weight traffic, whose every position reads the whole network.
+    Synchronises."""
+    L = load_library()
+    nbytes = -(-int(nbytes) // 32768) * 32768
+    buf = torch.zeros(nbytes // 4, dtype=torch.int32, device=device)
+    sink = torch.zeros(64, dtype=torch.int32, device=device)
+    with torch.cuda.device(buf.device):
+        rate = L.bf_stream_rate(buf.data_ptr(), nbytes, workgroups, reps, sink.data_ptr(),
+                                torch.cuda.current_stream().cuda_stream)
+    if rate < 0:
+        raise RuntimeError(f"bf_stream_rate: {L.bf_last_error().decode()}")
     return float(rate)
 
 

@@ -237,6 +237,17 @@ double bf_time_kernel_ms(const bf_eval_args* args, void* stream, int warmup, int
  * docs/ledger/perf.md:616-642). */
 double bf_mfma_rate(int quant, int* scratch, int iters, int reps, void* stream);
 
+/* Measured rate, in TB/s, at which the compute units can stream one buffer out of the cache
+ * hierarchy when every workgroup reads all of it -- the access pattern of the evaluator's weights
+ * (each position's workgroup reads the whole network; the kernels' weight traffic is priced
+ * against this number).  `workgroups` workgroups of four wavefronts each read `bytes` (a multiple
+ * of 32768) from the DEVICE buffer `buf`, wavefront w its quarter, 16 bytes per lane and load,
+ * eight loads in flight, from staggered starting offsets; `reps` timed launches after one
+ * warm-up launch; `sink` is a DEVICE buffer of 256 bytes that is never written for a buffer of
+ * equal 32-bit words.  Returns a negative bf_status on error.  Synchronises the stream.
+ * No counterpart in the reference. */
+double bf_stream_rate(const void* buf, size_t bytes, int workgroups, int reps, int* sink, void* stream);
+
 /* In-kernel phase accounting, the counterpart of the reference's profile hooks
  * (reference csrc/encoder.cu:1083-1177 and :1886-1903: set_profile / read_profile /
  * profile_phases).  bf_profile_phases runs a separately compiled build of the kernel the

@@ -42,6 +42,7 @@ int main(void) {
     if (bf_movegen(NULL, NULL, 4, NULL, NULL, NULL) != BF_ERR_ARGUMENT) return 13;
     if (bf_compact_leaves(NULL, 4, NULL, NULL, NULL) != BF_ERR_ARGUMENT) return 17;
     if (bf_mfma_rate(BF_QUANT_INT8, NULL, 10, 1, NULL) >= 0.0) return 14;
+    if (bf_stream_rate(NULL, 32768, 4, 1, NULL, NULL) >= 0.0) return 18;
     printf("abi ok: %s\n", bf_last_error());
     return 0;
 }

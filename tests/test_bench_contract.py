@@ -50,3 +50,4 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert par["bit_exact_vs_c_checker"] is True and par["masked_argmax_equal"] is True
     assert par["prior_space_vs_int8_emulation"]["max_abs"] < 1e-2 and par["prior_space_vs_int8_emulation"]["edge_set_differs"] == 0
     assert r["weight_stream"]["bytes_per_launch"] == 4096 * 6_455_296
+    assert r["weight_stream"]["achieved_TBps"] < 1.1 * r["weight_stream"]["stream_ceiling_TBps"] < 1.1 * r["weight_stream"]["l1_fill_nominal_TBps"]

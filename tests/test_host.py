@@ -77,6 +77,9 @@ def test_null_arguments_are_rejected_without_a_launch():
     # the matrix-pipe probe rejects a missing buffer and a bad format before touching a device
     assert lib.bf_mfma_rate(0, None, 10, 1, None) == -1.0
     assert lib.bf_mfma_rate(7, ctypes.c_void_p(4096), 10, 1, None) == -1.0
+    # so does the weight-stream probe: no buffer, a size that is not whole groups of loads
+    assert lib.bf_stream_rate(None, 32768, 4, 1, ctypes.c_void_p(4096), None) == -1.0
+    assert lib.bf_stream_rate(ctypes.c_void_p(4096), 1000, 4, 1, ctypes.c_void_p(4096), None) == -1.0
 
 
 def test_kernel_choice_follows_shape_blobs_and_batch_size():

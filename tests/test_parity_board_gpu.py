@@ -386,6 +386,14 @@ def test_matrix_pipe_probe_reports_a_plausible_rate():
         assert 1000.0 < rate < 5500.0, (fmt, rate)
 
 
+def test_weight_stream_probe_reports_a_plausible_rate():
+    # a buffer that fits every L2 streams faster than one the size of the 512-wide network (50 MB,
+    # more than the L2s hold); both lie between HBM speed and the L1 fill paths' nominal 39 TB/s
+    from brokefish_amd.hip_impl import stream_rate
+    small, large = stream_rate(1 << 20, workgroups=2048), stream_rate(50_626_560, workgroups=1024, reps=1)
+    assert 8.0 < small < 45.0 and 2.0 < large < small, (small, large)
+
+
 @pytest.mark.parametrize("kernel,n", [("auto", 64), ("auto", 1000), ("quad", 64)])
 def test_phase_profile_runs_on_the_kernel_the_call_selects_and_leaves_the_outputs_right(kernel, n):
     torch.manual_seed(0)
