@@ -110,6 +110,9 @@ def main() -> int:
     ap.add_argument("--copy-probe-mib", type=int, default=0,
                     help="also run one device copy of this many MiB (a kernel of known HBM traffic, "
                          "to calibrate FETCH_SIZE / WRITE_SIZE counter runs)")
+    ap.add_argument("--phases", action="store_true",
+                    help="add `phases` to the line: shader-clock ticks per wavefront and phase from the profiling "
+                         "build of the selected kernel (int8, kernels twin / octo / quad)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this path runs on one GPU (positions shard with no exchange step); --gpus must be 1",
@@ -189,6 +192,10 @@ def main() -> int:
     # MFMA chains, no memory traffic), next to the datasheet peak that `frac` is quoted against
     from brokefish_amd.hip_impl import mfma_rate
     line["roofline"]["measured_mfma_rate"] = mfma_rate(a.quant)
+    if a.phases:
+        ph = model.profile_phases(bd, cd, rd, md)
+        line["phases"] = {"kernel": kname, "ticks_per_wavefront": {k: round(v, 1) for k, v in ph.items()},
+                          "share_of_total": {k: round(v / ph["total"], 4) for k, v in ph.items() if k != "total"}}
     del model, bd, cd, rd, md
     if headline and not a.no_extras:
         # configuration 3: the batch sweep (small-batch latency regime), same net, same generator
