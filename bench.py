@@ -28,9 +28,9 @@ PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s
 PEAK_FP16_OPS = 2.5e15                # dense fp16 MFMA: the e4m3 format's products run on the fp16 instruction
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/
 # (calibrated on a 1 GiB copy), by (network shape, kernel, batch).
-MEASURED_TRAFFIC_BYTES = {("base", "twin", 4096): 0.81e9, ("base", "quad", 4096): 3.07e9,
+MEASURED_TRAFFIC_BYTES = {("base", "twin", 4096): 0.78e9, ("base", "quad", 4096): 3.07e9,
                           ("base", "board", 256): 5.5e7, ("base", "octo", 256): 5.5e7, ("stress", "board", 16384): 2.66e10,
-                          ("stress", "octo", 16384): 3.36e10}
+                          ("stress", "octo", 16384): 3.61e10}
 MEASURED_TRAFFIC_BYTES_E4M3 = {("base", "twin", 4096): 0.97e9}
 
 
@@ -159,7 +159,8 @@ def main() -> int:
     peak = PEAK_FP16_OPS if fp8 else PEAK_INT8_OPS
     kname = model.kernel_choice(a.batch)
     traffic = (MEASURED_TRAFFIC_BYTES_E4M3 if fp8 else MEASURED_TRAFFIC_BYTES).get((a.shape, kname, a.batch))
-    weight_bytes = (50_626_560 if stress else 6_455_296) * a.batch      # each position streams its own copy from L2
+    # each position's workgroup streams its own copy of the weights from L2 (four positions share one in the quad kernel)
+    weight_bytes = 6_389_760 * ((a.batch + 3) // 4) if kname == "quad" else (50_626_560 if stress else 6_455_296) * a.batch
     line = {
         "metric": (f"network evals/sec at batch {a.batch} int8, 16-layer width-512 stress shape, on 1 MI355X" if stress
                    else f"network evals/sec at batch 4096 {'fp8 e4m3' if fp8 else 'int8'} on 1 MI355X"),
@@ -186,7 +187,7 @@ def main() -> int:
                                        "l1_fill_nominal_TBps": 256 * 64 * 2.4e9 / 1e12}},
     }
     from brokefish_amd.hip_impl import stream_rate
-    line["roofline"]["weight_stream"]["stream_ceiling_TBps"] = stream_rate(weight_bytes // a.batch, workgroups=min(a.batch, 4096),
+    line["roofline"]["weight_stream"]["stream_ceiling_TBps"] = stream_rate(6_389_760 if kname == "quad" else weight_bytes // a.batch, workgroups=min(a.batch, 4096),
                                                                            reps=1 if stress else 3)
     # the matrix pipe's measured ceiling for the instruction the kernel uses (register-resident
     # MFMA chains, no memory traffic), next to the datasheet peak that `frac` is quoted against
