@@ -216,6 +216,11 @@ def test_full_batch_properties_at_4096(setup):
         emu = emulated.forward(sd, b[idx], c[idx], r[idx], mode="e4m3")
         f32 = emulated.forward(sd, b[idx], c[idx], r[idx], mode="fp32")
     raw = model.forward_full(bd, cd, rd)[0][idx.cuda()].cpu()
-    assert ((raw - emu[0]).abs().reshape(64, -1).amax(1) <= 2e-2).float().mean() > 0.5
+    # boards whose free-running logits stay within the 2e-2 target: every board that flips no byte at an
+    # e4m3 tie (test above) does; measured 61 % of these 64 boards on this per-layer-distinct network (88-89 % on
+    # the seed-0 network), and two orderings of the torch emulation agree with each other on 84-93 %
+    within = ((raw - emu[0]).abs().reshape(64, -1).amax(1) <= 2e-2).float().mean().item()
+    print(f"\n  e4m3 at batch 4096: {within:.0%} of 64 sampled boards within 2e-2 of the emulation free-running")
+    assert within >= 0.55
     assert (raw - f32[0]).abs().mean() < 1.15 * (emu[0] - f32[0]).abs().mean()
     assert (raw - emu[0]).abs().max() < (emu[0] - f32[0]).abs().max()
