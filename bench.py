@@ -30,7 +30,7 @@ PEAK_FP16_OPS = 2.5e15                # dense fp16 MFMA: the e4m3 format's produ
 # (calibrated on a 1 GiB copy), by (network shape, kernel, batch).
 MEASURED_TRAFFIC_BYTES = {("base", "twin", 4096): 0.78e9, ("base", "quad", 4096): 3.07e9,
                           ("base", "board", 256): 5.5e7, ("base", "octo", 256): 5.5e7, ("stress", "board", 16384): 2.66e10,
-                          ("stress", "octo", 16384): 3.61e10}
+                          ("stress", "octo", 16384): 2.95e10}
 MEASURED_TRAFFIC_BYTES_E4M3 = {("base", "twin", 4096): 0.97e9}
 
 

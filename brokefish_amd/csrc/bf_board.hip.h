@@ -83,17 +83,21 @@ struct Cfg : Layout<DM> {
     static constexpr int RING_BYTES = TWIN ? 0 : 4 * L::SLOTS * BLOCK;
     static constexpr int XCH_OFF = RING_BYTES;
     static constexpr int HID_OFF = XCH_OFF + 3 * (NW / 4) * FRAG;
-    // the quantised hidden row of the feed-forward block: the whole row (32 tiles) for the 256-wide
-    // network, one step of 512 channels (16 tiles) for the 512-wide one, whose row does not fit
-    static constexpr bool FULLHID = DM == 256;
+    // the quantised hidden row of the feed-forward block: the whole row (F / 32 tiles) where it fits
+    // -- the 256-wide network (32 KiB), and the 512-wide one (64 KiB) with eight wavefronts, no
+    // weight ring and one parameter copy per quarter; otherwise one step of 512 channels (16 tiles)
+    static constexpr bool FULLHID = DM == 256 || (OCTO && DM == 512);
     static constexpr int HID_FRAGS = FULLHID ? L::F / 32 : 16;
     static constexpr int ACT_OFF = HID_OFF + HID_FRAGS * FRAG;
     static constexpr int PAR_OFF = ACT_OFF + L::NT * FRAG;
     // three workgroups per compute unit: only the often-read part of the feed-forward parameters
     // is kept in LDS, the rest is read from global memory where it is used
     static constexpr bool BTAIL_GLOBAL = TWIN && !OCTO && BF_TWIN_OCC >= 3;
-    static constexpr int PWL_FLOATS = L::A_FLOATS + (BTAIL_GLOBAL ? L::B_LDS_FLOATS : L::B_FLOATS);   // per wave, in LDS
-    static constexpr int LDS_BYTES = PAR_OFF + NW * PWL_FLOATS * 4;
+    static constexpr int PWL_FLOATS = L::A_FLOATS + (BTAIL_GLOBAL ? L::B_LDS_FLOATS : L::B_FLOATS);   // per copy, in LDS
+    // four wavefronts: every wave keeps its own copy of its quarter's parameters (no wave waits for
+    // another's transfer).  Eight: the two waves of a quarter share one copy, fetched by the first.
+    static constexpr int PAR_COPIES = 4;
+    static constexpr int LDS_BYTES = PAR_OFF + PAR_COPIES * PWL_FLOATS * 4;
     static_assert(!OCTO || TWIN, "eight wavefronts per position take their weights straight to registers");
     static_assert(LDS_BYTES <= (TWIN && !OCTO ? 160 / BF_TWIN_OCC : 160) * 1024, "LDS budget: one or two workgroups per compute unit");
     static_assert(L::NT * 4 * FRAG <= LDS_BYTES - HID_OFF, "normalised stream overlay");
@@ -227,11 +231,13 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     constexpr int HT = 4 / SUB;               // hidden tiles a wave computes per feed-forward step
     constexpr int NB = BPW / SUB;             // weight blocks a wave consumes per layer
     // register sets of the prefetch: NSETS - 1 half-blocks in flight
-    constexpr int NSETS = OCTO ? BF_OCTO_SETS : BF_TWIN_SETS;
+    // (the 512-wide network's eight-wave form: three sets measure the same as four and spill
+    // 15 registers instead of 26)
+    constexpr int NSETS = OCTO ? (DM == 512 ? 3 : BF_OCTO_SETS) : BF_TWIN_SETS;
     static_assert(TW % SUB == 0 && (2 * NB) % NSETS == 0, "tiles and register sets must split evenly");
     constexpr bool FULLHID = C::FULLHID;      // the whole quantised hidden row stays in LDS
     static_assert(block_at_covers_layer<KC, TW, SUB, BPW, FULLHID>(), "block_at must enumerate a layer's blocks exactly once");
-    static_assert(!FULLHID || (STEPS == 2 && STEPS == TW && KCF == 2 * STEPS), "the full-row form is laid out for the 256-wide network");
+    static_assert(!FULLHID || (STEPS == TW && KCF == 2 * STEPS), "the full-row form: as many steps as tiles per quarter, two k-chunks per step");
     static_assert(SLOTS <= HB && NSETS - 1 <= 2 * HB + 2, "the first prefetches of a heads-only run stay inside the head blocks");
     constexpr int XS = NW * 64;               // floats of one exchange slot
     // Eight wavefronts on the 512-wide network: a wave has 256 registers and the quantised row alone
@@ -304,7 +310,12 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
     float* const xch = reinterpret_cast<float*>(lds + C::XCH_OFF);
     uint8_t* const hid = lds + C::HID_OFF;
     uint8_t* const act = lds + C::ACT_OFF;
-    float* const pA = reinterpret_cast<float*>(lds + C::PAR_OFF) + wave * C::PWL_FLOATS;   // every wave keeps its own copy
+    // the quarter's side parameters in LDS: with four waves the wave's own copy; with eight one copy
+    // per quarter, transferred by the quarter's first wave at points where a workgroup barrier
+    // separates the transfer from the other wave's last read of the old and first read of the new
+    constexpr bool SHARED_PAR = OCTO;
+    const bool par_owner = !SHARED_PAR || sub == 0;
+    float* const pA = reinterpret_cast<float*>(lds + C::PAR_OFF) + q * C::PWL_FLOATS;
     constexpr int B_COPY = C::BTAIL_GLOBAL ? C::B_LDS_FLOATS : C::B_FLOATS;
     float* const pB = pA + C::A_FLOATS;
     // the quarter's weight stream, from the first layer that runs; block `seq` in the quarter's order
@@ -482,7 +493,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
         for (int j = 0; j < SLOTS; j++) issue_block(j, j);   // layer blocks, or the first head blocks (SLOTS <= HB)
     }
-    if (nl_run > 0) {
+    if (nl_run > 0 && par_owner) {
         dma(wpar + (size_t)a.l0 * C::PW_FLOATS, pA, C::A_FLOATS, lane);
         dma(wpar + (size_t)a.l0 * C::PW_FLOATS + C::A_FLOATS, pB, B_COPY, lane);
     }
@@ -587,6 +598,11 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             float y[TWW][16];
             layernorm(x, pA + C::A_LN1G + 32 * t0, pA + C::A_LN1B + 32 * t0, y);
             quant_exchange(y, sa, xq, TAPS ? a.taps.qa_qkv : nullptr, bl);
+        }
+        // a shared copy's feed-forward parameters of this layer (the first layer's came with the start)
+        if (SHARED_PAR && par_owner && li > 0) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            dma(wpar + (size_t)l * C::PW_FLOATS + C::A_FLOATS, pB, B_COPY, lane);
         }
         BF_PHASE(PH_LN1);
         float sa_tok[KC][16];   // activation scale of token ch(r, g), for the V tiles whose rows are tokens
@@ -733,15 +749,22 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
             }
         }
         BF_PHASE(PH_OUT);
-        // the attention-phase parameters are dead: fetch the next layer's
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        dma(wpar + (size_t)lnext * C::PW_FLOATS, pA, C::A_FLOATS, lane);
+        // the attention-phase parameters are dead for this wave: fetch the next layer's (a shared
+        // copy: after the next barriers, which the quarter's other wave reaches when it is done too)
+        if constexpr (!SHARED_PAR) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            dma(wpar + (size_t)lnext * C::PW_FLOATS, pA, C::A_FLOATS, lane);
+        }
 
         // ---- feed-forward --------------------------------------------------------------------------------
         {
             float y[TWW][16];
             layernorm(x, pB + C::B_LN2G + 32 * t0, pB + C::B_LN2B + 32 * t0, y);
             quant_exchange(y, sa, xq, TAPS ? a.taps.qa_ff1 : nullptr, bl);
+        }
+        if (SHARED_PAR && par_owner) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            dma(wpar + (size_t)lnext * C::PW_FLOATS, pA, C::A_FLOATS, lane);
         }
         BF_PHASE(PH_LN2);
         constexpr int KF = 3 * KC * TWW + KC * TWW;   // the wave's first feed-forward block of the layer
@@ -1065,8 +1088,10 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                     }
             }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        dma(wpar + (size_t)lnext * C::PW_FLOATS + C::A_FLOATS, pB, B_COPY, lane);
+        if constexpr (!SHARED_PAR) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            dma(wpar + (size_t)lnext * C::PW_FLOATS + C::A_FLOATS, pB, B_COPY, lane);
+        }
         BF_PHASE(PH_FF2);
 #undef BF_WMM
 #undef BF_WMM_FROM
