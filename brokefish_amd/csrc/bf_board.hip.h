@@ -14,8 +14,7 @@
 // Three forms, selected by TWIN and OCTO, with identical results:
 //   TWIN = false  one workgroup per compute unit, 512 registers per wave.  Weight blocks stream
 //                 through a private LDS ring per wave (direct-to-LDS loads, SLOTS blocks deep),
-//                 attention is software-pipelined across heads.  The only form the 512-wide
-//                 network fits.
+//                 attention is software-pipelined across heads.
 //   TWIN = true   two workgroups per compute unit: at most 80 KiB of LDS and 256 registers per
 //                 wave, so every SIMD holds two wavefronts of different positions and one's
 //                 waits (LDS round trips, barriers, MFMA results) are covered by the other's
@@ -30,9 +29,11 @@
 //                 per position (launches of up to one position per compute unit).
 //
 // LDS map (bytes): [ring: 4 waves x SLOTS x 8 KiB, absent in the TWIN form] [xch: 3 slots of
-// 64 floats per wave] [hid: 32 KiB (width 256: the whole hidden row) or 16 KiB (width 512: one
-// step)] [act: NT KiB] [par: PW floats per wave].  During the heads the
-// normalised stream (NT*4 KiB, fp32) overlays hid/act/par.
+// 64 floats per wave] [hid: the whole quantised hidden row (32 KiB at width 256, 64 KiB at width
+// 512 with eight wavefronts) or one step of it (16 KiB: width 512 with the weight ring)]
+// [act: NT KiB] [par: one copy of each quarter's side parameters -- the wave's own with four
+// wavefronts, shared by the quarter's two with eight].  During the heads the normalised stream
+// (NT*4 KiB, fp32) overlays hid/act/par.
 #pragma once
 
 #include <atomic>
