@@ -51,3 +51,15 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert par["prior_space_vs_int8_emulation"]["max_abs"] < 1e-2 and par["prior_space_vs_int8_emulation"]["edge_set_differs"] == 0
     assert r["weight_stream"]["bytes_per_launch"] == 4096 * 6_455_296
     assert r["weight_stream"]["achieved_TBps"] < 1.1 * r["weight_stream"]["stream_ceiling_TBps"] < 1.1 * r["weight_stream"]["l1_fill_nominal_TBps"]
+
+
+@pytest.mark.gpu
+def test_phase_profile_flag_adds_the_phases_of_the_selected_kernel():
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--no-cpu", "--no-extras", "--batch", "256",
+                          "--steps", "2", "--warmup", "1", "--phases"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    d = json.loads([l for l in run.stdout.splitlines() if l.strip()][-1])
+    ph = d["phases"]
+    assert ph["kernel"] == "octo" and ph["ticks_per_wavefront"]["total"] > 0
+    parts = [v for k, v in ph["share_of_total"].items() if k != "sync_wait"]     # barrier time is inside the phases
+    assert 0.95 < sum(parts) < 1.05 and 0.0 < ph["share_of_total"]["sync_wait"] < 0.5
