@@ -100,7 +100,7 @@ def main() -> int:
     ap.add_argument("--shape", choices=("base", "stress"), default="base",
                     help="base: 8 layers, width 256 (the headline metric); stress: 16 layers, width 512, "
                          "16 heads, default batch 16384")
-    ap.add_argument("--kernel", choices=("auto", "quad", "board", "twin", "octo"), default="auto",
+    ap.add_argument("--kernel", choices=("auto", "quad", "board", "twin", "octo", "duo"), default="auto",
                     help="four positions per workgroup; one position per workgroup with one (board; octo: eight wavefronts) or two (twin) workgroups per compute unit; auto: by batch size")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=64)

@@ -18,8 +18,9 @@
 //
 // Arithmetic contract (what the CPU checker restates operation by operation):
 //   embedding  ((sq + ts) + ct) + (clock + rep)                        fp32
-//   LayerNorm  per lane half four group sums (a quarter of the tiles each, sequential over
-//              tiles then r) added in group order, then the two halves
+//   LayerNorm  per lane half: every 32-wide tile's 16 values form one chain from zero; the tile
+//              sums of a quarter of the width are added as a balanced tree (t0 + t1, or
+//              (t0 + t1) + (t2 + t3)); the four quarter sums are added in order; then the two halves
 //   quantise   s = amax / qmax, q = rint(x / s)  (x / s as a correctly rounded quotient)
 //   GEMM       exact int32; descale fl(fl(acc * sa) * sw) + b; several k-chunks are summed
 //              in fp64 before the single cast to fp32
@@ -152,9 +153,16 @@ hipError_t launch_octo256_fp8(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo256_fp8_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512_taps(const KArgs& k, hipStream_t stream);
+// two positions per workgroup of eight wavefronts (256-wide network): a weight fragment fetched
+// once serves both positions
+hipError_t launch_duo256(const KArgs& k, hipStream_t stream);
+hipError_t launch_duo256_taps(const KArgs& k, hipStream_t stream);
+hipError_t launch_duo256_fp8(const KArgs& k, hipStream_t stream);
+hipError_t launch_duo256_fp8_taps(const KArgs& k, hipStream_t stream);
 // the int8 builds that carry the phase profile
 hipError_t launch_twin256_prof(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo256_prof(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_duo256_prof(const KArgs& k, hipStream_t stream);
 
 }  // namespace bf

@@ -369,47 +369,48 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
         for (int s = 0; s < 8; s++) fr[s] = *reinterpret_cast<const v4i*>(&myring[slot * BLOCK + s * FRAG + lane * 16]);
     };
-    // Row sum over the width: `chain(start)` adds this wave's values to `start` one by one; a
-    // quarter's values form one chain (with eight waves the quarter's second wave continues the
-    // first one's), and the four quarter sums are added in order.
-    // Four waves: one exchange slot per call site (`slot`), so that a fast wave's next partial
-    // cannot overwrite what a slow wave still reads.  Eight waves: slots 0 and 1 serve every call;
-    // the two barriers of a call separate its traffic from the previous call's.
-    auto xsum = [&](auto&& chain, int slot) -> float {
-        if constexpr (!OCTO) {
-            xch[slot * XS + wave * 64 + lane] = chain(0.0f);
-            barrier();
-            const float* p = xch + slot * XS + lane;
-            return ((p[0] + p[64]) + p[128]) + p[192];
-        } else {
-            if (sub == 0) xch[q * 64 + lane] = chain(0.0f);
-            barrier();
-            if (sub == 1) xch[XS + q * 64 + lane] = chain(xch[q * 64 + lane]);
-            barrier();
-            const float* p = xch + XS + lane;
-            return ((p[0] + p[64]) + p[128]) + p[192];
-        }
+    // Row sum over the width.  Every tile's 16 values form one chain from zero; a wave adds the sums
+    // of its own tiles as a balanced tree and publishes the result; with eight waves the two halves
+    // of a quarter are added, then the four quarter sums in order -- the same tree whichever way
+    // the width is split over waves.  One exchange slot per call site (`slot`), so that a fast
+    // wave's next partial cannot overwrite what a slow wave still reads: between two uses of a
+    // slot lies at least one other workgroup barrier.
+    auto tiles_sum = [&](const float (&ts)[TWW]) -> float {
+        static_assert(TWW == 1 || TWW == 2 || TWW == 4, "tile sums are added as a balanced tree");
+        if constexpr (TWW == 1) return ts[0];
+        else if constexpr (TWW == 2) return ts[0] + ts[1];
+        else return (ts[0] + ts[1]) + (ts[2] + ts[3]);
+    };
+    auto xsum = [&](float part, int slot) -> float {
+        xch[slot * XS + wave * 64 + lane] = part;
+        barrier();
+        const float* p = xch + slot * XS + lane;
+        if constexpr (!OCTO) return ((p[0] + p[64]) + p[128]) + p[192];
+        else return (((p[0] + p[256]) + (p[64] + p[320])) + (p[128] + p[384])) + (p[192] + p[448]);
     };
     // LayerNorm of this wave's channels; gamma / beta point at this wave's slice
     auto layernorm = [&](const float (&x)[TWW][16], const float* gamma, const float* beta, float (&y)[TWW][16]) {
-        const float s = xsum([&](float acc) {
+        float ts[TWW];
 #pragma unroll
-            for (int i = 0; i < TWW; i++)
+        for (int i = 0; i < TWW; i++) {
+            float acc = 0.0f;
 #pragma unroll
-                for (int r = 0; r < 16; r++) acc = acc + x[i][r];
-            return acc;
-        }, 0);
+            for (int r = 0; r < 16; r++) acc = acc + x[i][r];
+            ts[i] = acc;
+        }
+        const float s = xsum(tiles_sum(ts), 0);
         const float mean = (s + partner(s, g)) * (1.0f / D);
-        const float v = xsum([&](float acc) {
 #pragma unroll
-            for (int i = 0; i < TWW; i++)
+        for (int i = 0; i < TWW; i++) {
+            float acc = 0.0f;
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const float d = x[i][r] - mean;
-                    acc = __builtin_fmaf(d, d, acc);
-                }
-            return acc;
-        }, 1);
+            for (int r = 0; r < 16; r++) {
+                const float d = x[i][r] - mean;
+                acc = __builtin_fmaf(d, d, acc);
+            }
+            ts[i] = acc;
+        }
+        const float v = xsum(tiles_sum(ts), 1);
         const float var = (v + partner(v, g)) * (1.0f / D);
         const float rstd = 1.0f / __builtin_sqrtf(var + a.eps);
 #pragma unroll

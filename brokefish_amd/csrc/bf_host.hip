@@ -106,6 +106,7 @@ static int choose_kernel(const bf_eval_args* a) {
     const bool board_can = have_board && (a->quant == BF_QUANT_INT8 || shape_ok(&a->shape));
     const bool twin_can = have_board && shape_ok(&a->shape);
     const bool octo_can = board_can;   // the same networks and formats as BOARD
+    const bool duo_can = twin_can;     // the 256-wide network, both formats
     switch (a->kernel) {
     case BF_KERNEL_QUAD:
         if (!quad_can) return fail(BF_ERR_UNSUPPORTED, "the four-positions-per-workgroup kernel needs the 256-wide network and wstream/fparams");
@@ -121,6 +122,10 @@ static int choose_kernel(const bf_eval_args* a) {
         if (!octo_can)
             return fail(BF_ERR_UNSUPPORTED, "the eight-wavefronts-per-position kernel needs board_wstream/board_fparams (512-wide network: the int8 format)");
         return BF_KERNEL_OCTO;
+    case BF_KERNEL_DUO:
+        if (!duo_can)
+            return fail(BF_ERR_UNSUPPORTED, "the two-positions-per-workgroup kernel needs the 256-wide network and board_wstream/board_fparams");
+        return BF_KERNEL_DUO;
     case BF_KERNEL_AUTO:
         if (octo_can) return (twin_can && a->n > kBoardMaxN) ? BF_KERNEL_TWIN : BF_KERNEL_OCTO;
         if (quad_can) return BF_KERNEL_QUAD;
@@ -128,7 +133,7 @@ static int choose_kernel(const bf_eval_args* a) {
                         ? "the 512-wide network runs on the one-position-per-workgroup kernel: int8, board_wstream/board_fparams required"
                         : "wstream/fparams must not be NULL");
     default:
-        return fail(BF_ERR_ARGUMENT, "kernel must be BF_KERNEL_AUTO, BF_KERNEL_QUAD, BF_KERNEL_BOARD, BF_KERNEL_TWIN or BF_KERNEL_OCTO");
+        return fail(BF_ERR_ARGUMENT, "kernel must be BF_KERNEL_AUTO, BF_KERNEL_QUAD, BF_KERNEL_BOARD, BF_KERNEL_TWIN, BF_KERNEL_OCTO or BF_KERNEL_DUO");
     }
 }
 
@@ -137,7 +142,7 @@ extern "C" int bf_kernel_choice(const bf_eval_args* args) { return choose_kernel
 static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     *kind = choose_kernel(a);
     if (*kind < 0) return *kind;
-    const bool board = *kind == BF_KERNEL_BOARD || *kind == BF_KERNEL_TWIN || *kind == BF_KERNEL_OCTO;
+    const bool board = *kind == BF_KERNEL_BOARD || *kind == BF_KERNEL_TWIN || *kind == BF_KERNEL_OCTO || *kind == BF_KERNEL_DUO;
     if (a->n < 1 || a->n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
     if (!a->boards || !a->control || !a->rep) return fail(BF_ERR_ARGUMENT, "boards/control/rep must not be NULL");
     if (!a->policy || !a->promo || !a->value) return fail(BF_ERR_ARGUMENT, "policy/promo/value must not be NULL");
@@ -159,7 +164,7 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     if (a->value_mode < BF_VALUE_KING || a->value_mode > BF_VALUE_PRENORM)
         return fail(BF_ERR_ARGUMENT, "value_mode must be BF_VALUE_KING, BF_VALUE_POOLED or BF_VALUE_PRENORM");
     if (a->value_mode != BF_VALUE_KING && !board)
-        return fail(BF_ERR_UNSUPPORTED, "the pooled value heads run on the one-position-per-workgroup kernels (BOARD, TWIN, OCTO)");
+        return fail(BF_ERR_UNSUPPORTED, "the pooled value heads run on the BOARD, TWIN, OCTO and DUO kernels");
     if (!board && (!a->workspace || ((uintptr_t)a->workspace & 15) || a->workspace_bytes < bf_workspace_bytes(&a->shape, a->n)))
         return fail(BF_ERR_ARGUMENT, "workspace must be 16-byte aligned and hold bf_workspace_bytes(shape, n) bytes");
     memset(k, 0, sizeof(*k));
@@ -221,6 +226,13 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream
             e = a->taps ? bf::launch_octo256_fp8_taps(k, stream) : bf::launch_octo256_fp8(k, stream);
         else
             e = a->taps ? bf::launch_octo256_taps(k, stream) : bf::launch_octo256(k, stream);
+    } else if (kind == BF_KERNEL_DUO) {
+        if (k.profile)
+            e = bf::launch_duo256_prof(k, stream);
+        else if (a->quant == BF_QUANT_E4M3)
+            e = a->taps ? bf::launch_duo256_fp8_taps(k, stream) : bf::launch_duo256_fp8(k, stream);
+        else
+            e = a->taps ? bf::launch_duo256_taps(k, stream) : bf::launch_duo256(k, stream);
     } else if (kind == BF_KERNEL_TWIN) {
         if (k.profile)
             e = bf::launch_twin256_prof(k, stream);
@@ -229,7 +241,7 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream
         else
             e = a->taps ? bf::launch_twin256_taps(k, stream) : bf::launch_twin256(k, stream);
     } else if (kind == BF_KERNEL_BOARD) {
-        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the TWIN, OCTO and QUAD kernels");
+        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the TWIN, OCTO, DUO and QUAD kernels");
         if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_board512_taps(k, stream) : bf::launch_board512(k, stream);
         else if (a->quant == BF_QUANT_E4M3)
@@ -322,7 +334,7 @@ extern "C" int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_
     if (rc) return rc;
     if (args->taps) return fail(BF_ERR_ARGUMENT, "the phase profile runs without taps");
     if (args->quant != BF_QUANT_INT8) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the int8 format only");
-    if (kind == BF_KERNEL_BOARD) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the TWIN, OCTO and QUAD kernels");
+    if (kind == BF_KERNEL_BOARD) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the TWIN, OCTO, DUO and QUAD kernels");
     if (!cycles) return fail(BF_ERR_ARGUMENT, "cycles must not be NULL");
     k.profile = reinterpret_cast<unsigned long long*>(cycles);
     return launch(args, k, kind, (hipStream_t)stream);

@@ -76,31 +76,38 @@ __device__ __forceinline__ void load_frags(int blk, v4i (&fr)[8], Stream& st, in
 // LayerNorm of the residual rows, affine applied, in the fixed lane order; gamma/beta in LDS or global
 __device__ __forceinline__ void layernorm(const float (&x)[NT][16], const float* gamma, const float* beta,
                                           float eps, int g, float (&y)[NT][16]) {
-    // per lane: four group sums (a quarter of the tiles each, sequential over tiles then r),
-    // added in group order; then the two lanes of the token
+    // per lane: every tile's 16 values form one chain from zero, the two tile sums of a quarter of
+    // the width are added, the four quarter sums are added in order; then the two lanes of the token
+    static_assert(NT == 8, "two tiles per quarter of the width");
     float sg[4];
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        float s = 0.0f;
+        float ts[2];
 #pragma unroll
-        for (int n = q * (NT / 4); n < (q + 1) * (NT / 4); n++)
+        for (int n = 0; n < 2; n++) {
+            float s = 0.0f;
 #pragma unroll
-            for (int r = 0; r < 16; r++) s = s + x[n][r];
-        sg[q] = s;
+            for (int r = 0; r < 16; r++) s = s + x[2 * q + n][r];
+            ts[n] = s;
+        }
+        sg[q] = ts[0] + ts[1];
     }
     const float s = ((sg[0] + sg[1]) + sg[2]) + sg[3];
     const float mean = (s + partner(s, g)) * (1.0f / D);
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        float v = 0.0f;
+        float ts[2];
 #pragma unroll
-        for (int n = q * (NT / 4); n < (q + 1) * (NT / 4); n++)
+        for (int n = 0; n < 2; n++) {
+            float v = 0.0f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const float d = x[n][r] - mean;
+                const float d = x[2 * q + n][r] - mean;
                 v = __builtin_fmaf(d, d, v);
             }
-        sg[q] = v;
+            ts[n] = v;
+        }
+        sg[q] = ts[0] + ts[1];
     }
     const float v = ((sg[0] + sg[1]) + sg[2]) + sg[3];
     const float var = (v + partner(v, g)) * (1.0f / D);

@@ -534,7 +534,7 @@ class FusedEncoder:
 
     D, DFF, T, H = 256, 1024, 32, 8
     SHAPES = ((256, 1024, 8), (512, 2048, 16))     # (d_model, d_ff, heads) the library carries
-    KERNELS = {"auto": 0, "quad": 1, "board": 2, "twin": 3, "octo": 4}   # enum bf_kernel
+    KERNELS = {"auto": 0, "quad": 1, "board": 2, "twin": 3, "octo": 4, "duo": 5}   # enum bf_kernel
     ACC_DTYPES = ("fp16", "fp32")
     VALUE_HEADS = ("king", "pooled", "prenorm")     # brokefish/nn/model.py:89
     n_value = 1
@@ -579,7 +579,7 @@ class FusedEncoder:
             raise ValueError(f"value_head must be one of {self.VALUE_HEADS}, got {value_head!r}")
         if value_head != "king" and kernel == "quad":
             raise NotImplementedError("the pooled value heads run on the one-position-per-workgroup kernels "
-                                      "(kernel='auto', 'twin', 'octo' or 'board')")
+                                      "(kernel='auto', 'twin', 'duo', 'octo' or 'board')")
         # numbering of the reference class (brokefish/nn/cuda_impl.py:141-158): 0 king, 1 pooled, 2 prenorm
         self.value_head, self.vmode = value_head, self.VALUE_HEADS.index(value_head)
         layers = (net.encoder if net is not None else source).layers
@@ -605,7 +605,7 @@ class FusedEncoder:
             import warnings
             warnings.warn("FusedEncoder(net) without int8=True or fp8=True builds the int8 evaluator here; the "
                           "reference class builds its unquantised fp16 path for the same call", stacklevel=2)
-        if wide and kernel in ("quad", "twin"):
+        if wide and kernel in ("quad", "twin", "duo"):
             raise NotImplementedError("the 512-wide network runs on the one-position-per-workgroup kernels "
                                       "(kernel='octo', 'board' or 'auto') only")
         if not getattr(first, "norm_first", True) or getattr(first, "activation_relu_or_gelu", 1) != 1:
@@ -665,7 +665,8 @@ class FusedEncoder:
     def label(self) -> str:
         fmt = "e4m3" if self.fp8 else "int8"
         names = {"quad": "4 boards/workgroup", "board": "1 board/workgroup",
-                 "twin": "1 board/workgroup, 2 workgroups/CU", "octo": "1 board/workgroup of 8 wavefronts"}
+                 "twin": "1 board/workgroup, 2 workgroups/CU", "octo": "1 board/workgroup of 8 wavefronts",
+                 "duo": "2 boards/workgroup of 8 wavefronts"}
         if self.kernel != "auto":
             per = names[self.kernel]
         elif self.board_wstream is None:
@@ -739,7 +740,7 @@ class FusedEncoder:
         return a
 
     def kernel_choice(self, n: int) -> str:
-        """Which kernel a call with ``n`` positions runs ("quad", "board", "twin" or "octo")."""
+        """Which kernel a call with ``n`` positions runs ("quad", "board", "twin", "octo" or "duo")."""
         a = _Args()
         a.n, a.shape, a.quant, a.kernel = n, self._shape, (1 if self.fp8 else 0), self.KERNELS[self.kernel]
         a.wstream = a.fparams = 16 if self.wstream is not None else None        # only tested for NULL
@@ -747,7 +748,7 @@ class FusedEncoder:
         rc = self._lib.bf_kernel_choice(C.byref(a))
         if rc < 0:
             raise RuntimeError(f"bf_kernel_choice failed ({rc}): {self._lib.bf_last_error().decode()}")
-        return {1: "quad", 2: "board", 3: "twin", 4: "octo"}[rc]
+        return {1: "quad", 2: "board", 3: "twin", 4: "octo", 5: "duo"}[rc]
 
     def forward_expand(self, boards, control, rep, mask=None, max_edges: int = 96, active=None, out=None, leaves=None):
         """``forward_full`` followed on the same stream by the search's expand step
@@ -879,15 +880,15 @@ class FusedEncoder:
 
     def profile_phases(self, boards, control, rep, mask=None) -> Dict[str, float]:
         """Shader-clock cycles per phase, averaged over the wavefronts of one launch of the
-        profiling build of the kernel this call would run (TWIN, OCTO or QUAD, int8): the
+        profiling build of the kernel this call would run (TWIN, OCTO, DUO or QUAD, int8): the
         counterpart of the reference's read_profile / profile_phases.  ``sync_wait`` (time at
         workgroup barriers) is also contained in the phases around it; ``total`` is a wavefront's
         lifetime.  The outputs it writes are the normal ones."""
         n = self._check_inputs(boards, control, rep, mask)
         kind = self.kernel_choice(n)
         if self.fp8 or kind == "board":
-            raise NotImplementedError("the phase profile is built for the int8 format on the TWIN, OCTO and QUAD "
-                                      "kernels (kernel='auto', 'twin', 'octo' or 'quad')")
+            raise NotImplementedError("the phase profile is built for the int8 format on the TWIN, OCTO, DUO and QUAD "
+                                      "kernels (kernel='auto', 'twin', 'octo', 'duo' or 'quad')")
         self._ensure_full_buffers(n)
         k = self._lib.bf_profile_phase_count()
         cyc = torch.zeros(k, dtype=torch.int64, device=self.device)
@@ -900,7 +901,7 @@ class FusedEncoder:
         if rc:
             raise RuntimeError(f"bf_profile_phases failed ({rc}): {self._lib.bf_last_error().decode()}")
         torch.cuda.current_stream(self.device).synchronize()
-        waves = {"twin": 4 * n, "octo": 8 * n, "quad": 4 * ((n + 3) // 4)}[kind]
+        waves = {"twin": 4 * n, "octo": 8 * n, "duo": 8 * ((n + 1) // 2), "quad": 4 * ((n + 3) // 4)}[kind]
         return {self._lib.bf_profile_phase_name(i).decode(): cyc[i].item() / waves for i in range(k)}
 
     # -- debug taps (the counterpart of the reference's forward_stage) ------------

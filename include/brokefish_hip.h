@@ -40,7 +40,7 @@ enum bf_quant {
     BF_QUANT_E4M3 = 1
 };
 
-/* Four kernels compute the same function.
+/* Five kernels compute the same function.
  *   QUAD   four positions per workgroup, one wavefront each, weights shared through LDS; carries
  *          the phase profile (256-wide network, int8 and e4m3).
  *   BOARD  one position per workgroup, the four wavefronts split the model width; one workgroup
@@ -53,7 +53,10 @@ enum bf_quant {
  *          width, each taking half of the quarter's tiles), one workgroup per compute unit: the
  *          lowest latency per position for the 256-wide network, and the faster kernel for the
  *          512-wide one.
- * BOARD, TWIN and OCTO read the same blobs (board_wstream / board_fparams).  The 256-wide network
+ *   DUO    two positions per workgroup of eight wavefronts (the OCTO decomposition, every
+ *          wavefront doing its share for both positions), so that a weight fragment fetched from
+ *          L2 serves two positions (256-wide network, int8 and e4m3).
+ * BOARD, TWIN, OCTO and DUO read the same blobs (board_wstream / board_fparams).  The 256-wide network
  * runs in int8 and e4m3 on all four; the 512-wide network in int8 on OCTO and BOARD.  Kernels that
  * carry a network and a format return bit-identical results for it, so AUTO may pick by batch
  * size. */
@@ -62,7 +65,8 @@ enum bf_kernel {
     BF_KERNEL_QUAD = 1,
     BF_KERNEL_BOARD = 2,
     BF_KERNEL_TWIN = 3,
-    BF_KERNEL_OCTO = 4
+    BF_KERNEL_OCTO = 4,
+    BF_KERNEL_DUO = 5
 };
 
 enum bf_value_mode {

@@ -180,21 +180,33 @@ void bfo_int8_linear(const float* x, int m, int k, const float* w, int n, const 
 
 /* ---- LayerNorm in lane order -------------------------------------------------- */
 
+/* tile sums of a quarter of the width, added as a balanced tree (1, 2 or 4 tiles) */
+static float tree_sum(const float* ts, int n) {
+    if (n == 1) return ts[0];
+    if (n == 2) return ts[0] + ts[1];
+    return (ts[0] + ts[1]) + (ts[2] + ts[3]);
+}
+
 static void layernorm_rows(const float* x, int d, const float* gamma, const float* beta,
                            float eps, float* y) {
     for (int t = 0; t < T; t++) {
         const float* row = x + (size_t)t * d;
-        /* per lane half g: four group sums (a quarter of the tiles each, sequential over
-         * tiles then r) added in group order; then the two halves */
+        /* per lane half g: every 32-wide tile's 16 values form one chain from zero; the tile sums
+         * of a quarter of the width are added as a balanced tree (t0 + t1 for two tiles,
+         * (t0 + t1) + (t2 + t3) for four); the four quarter sums are added in order; then the
+         * two halves */
         const int tq = d / 32 / 4;
         float part[2];
         for (int g = 0; g < 2; g++) {
             float sg[4];
             for (int q = 0; q < 4; q++) {
-                float s = 0.0f;
-                for (int n = q * tq; n < (q + 1) * tq; n++)
-                    for (int r = 0; r < 16; r++) s = s + row[32 * n + ch(r, g)];
-                sg[q] = s;
+                float ts[4];
+                for (int n = 0; n < tq; n++) {
+                    float s = 0.0f;
+                    for (int r = 0; r < 16; r++) s = s + row[32 * (q * tq + n) + ch(r, g)];
+                    ts[n] = s;
+                }
+                sg[q] = tree_sum(ts, tq);
             }
             part[g] = ((sg[0] + sg[1]) + sg[2]) + sg[3];
         }
@@ -203,13 +215,16 @@ static void layernorm_rows(const float* x, int d, const float* gamma, const floa
         for (int g = 0; g < 2; g++) {
             float sg[4];
             for (int q = 0; q < 4; q++) {
-                float s = 0.0f;
-                for (int n = q * tq; n < (q + 1) * tq; n++)
+                float ts[4];
+                for (int n = 0; n < tq; n++) {
+                    float s = 0.0f;
                     for (int r = 0; r < 16; r++) {
-                        const float dv = row[32 * n + ch(r, g)] - mean;
+                        const float dv = row[32 * (q * tq + n) + ch(r, g)] - mean;
                         s = fmaf(dv, dv, s);
                     }
-                sg[q] = s;
+                    ts[n] = s;
+                }
+                sg[q] = tree_sum(ts, tq);
             }
             part[g] = ((sg[0] + sg[1]) + sg[2]) + sg[3];
         }
