@@ -28,20 +28,24 @@ PEAK_INT8_OPS = 5.0e15                # MI355X dense int8 MFMA, ops/s
 PEAK_FP16_OPS = 2.5e15                # dense fp16 MFMA: the e4m3 format's products run on the fp16 instruction
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/
 # (calibrated on a 1 GiB copy), by (network shape, kernel, batch).
-MEASURED_TRAFFIC_BYTES = {("base", "twin", 4096): 0.78e9, ("base", "quad", 4096): 3.07e9,
+MEASURED_TRAFFIC_BYTES = {("base", "duo", 4096): 0.445e9, ("base", "twin", 4096): 0.78e9, ("base", "quad", 4096): 3.07e9,
                           ("base", "board", 256): 5.5e7, ("base", "octo", 256): 5.5e7, ("stress", "board", 16384): 2.66e10,
                           ("stress", "octo", 16384): 2.95e10}
 MEASURED_TRAFFIC_BYTES_E4M3 = {("base", "twin", 4096): 0.97e9}
+# vector-ALU instructions per launch (SQ_INSTS_VALU of the same counter runs), by (network shape, kernel, batch):
+# with the matrix products hidden, the launch cannot be shorter than these instructions' issue time
+MEASURED_VALU_INSTS = {("base", "duo", 4096): 5.938e8, ("base", "twin", 4096): 5.513e8}
+SIMDS, CLOCK_HZ = 1024, 2.4e9
 
 
-def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0, mode: str = "int8"):
+def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0, mode: str = "int8", plies: int = 80):
     """The int8- (or e4m3-) simulated forward of oracle/emulated.py on the host cores (a port,
     not the reference's files, which do not travel)."""
     import torch
     from brokefish_amd import positions
     from oracle import emulated
     sd = {k: v.detach() for k, v in net.state_dict().items()}
-    b, c, r, m = positions.random_positions(batch, plies=120, seed=0)
+    b, c, r, m = positions.random_positions(batch, plies=plies, seed=0)   # configs[0]: playouts of 0-80 plies
     torch.set_num_threads(threads)
     with torch.no_grad():
         t0 = time.perf_counter()
@@ -56,7 +60,7 @@ def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0, mode: st
     times.sort()
     med = times[len(times) // 2]
     return {"value": batch / med, "unit": "evals/s", "cores": threads, "kind": "port",
-            "sample": f"{reps} reps of batch {batch} ({mode}-simulated PyTorch forward, median), "
+            "sample": f"{reps} reps of batch {batch}, seeded random playouts of 0-{plies} plies ({mode}-simulated PyTorch forward, median), "
                       f"os.cpu_count()={os.cpu_count()}"}
 
 
@@ -78,15 +82,6 @@ def physical_cores() -> int:
         return len(seen) or len(allowed)
     except OSError:
         return os.cpu_count() or 1
-
-
-def time_config(net, fmt, batch, kernel="auto", iters=20, warmup=3):
-    """(kernel ms per launch from HIP events on the launch stream, kernel name) for one configuration."""
-    from brokefish_amd import encoder_impl, positions
-    model = encoder_impl("hip")(net, fp8=True, kernel=kernel) if fmt == "e4m3" else encoder_impl("hip")(net, int8=True, kernel=kernel)
-    sb, sc, sr, sm = (t.cuda() for t in positions.random_positions(batch, plies=120, seed=0))
-    ms = model.time_kernel_ms(sb, sc, sr, sm, warmup=warmup, iters=iters)
-    return ms, model.kernel_choice(batch), model
 
 
 def main() -> int:
@@ -159,8 +154,10 @@ def main() -> int:
     peak = PEAK_FP16_OPS if fp8 else PEAK_INT8_OPS
     kname = model.kernel_choice(a.batch)
     traffic = (MEASURED_TRAFFIC_BYTES_E4M3 if fp8 else MEASURED_TRAFFIC_BYTES).get((a.shape, kname, a.batch))
-    # each position's workgroup streams its own copy of the weights from L2 (four positions share one in the quad kernel)
-    weight_bytes = 6_389_760 * ((a.batch + 3) // 4) if kname == "quad" else (50_626_560 if stress else 6_455_296) * a.batch
+    # each workgroup streams its own copy of the weights from L2
+    # (four positions share one copy in the quad kernel, two in the duo kernel)
+    weight_bytes = (6_389_760 * ((a.batch + 3) // 4) if kname == "quad" else 6_455_296 * ((a.batch + 1) // 2) if kname == "duo"
+                    else (50_626_560 if stress else 6_455_296) * a.batch)
     line = {
         "metric": (f"network evals/sec at batch {a.batch} int8, 16-layer width-512 stress shape, on 1 MI355X" if stress
                    else f"network evals/sec at batch 4096 {'fp8 e4m3' if fp8 else 'int8'} on 1 MI355X"),
@@ -178,6 +175,12 @@ def main() -> int:
                      # FETCH_SIZE + WRITE_SIZE counter result of the same command summarised under profiles/
                      "traffic": traffic, "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (not measured in this run)" if traffic else None,
                      "kernel_ms": kern_ms, "ops_per_launch": ops_per_eval * a.batch,
+                     # what the launch cannot go below with every matrix product hidden: the vector instructions
+                     # the bit-exact fp32 / fp64 epilogues, LayerNorm, softmax and quantisers take, at four clocks
+                     # each on 1024 SIMDs (instruction count from the counter runs under profiles/, like `traffic`)
+                     "valu_floor_ms": (MEASURED_VALU_INSTS[(a.shape, kname, a.batch)] * 4 / (SIMDS * CLOCK_HZ) * 1e3
+                                       if not fp8 and (a.shape, kname, a.batch) in MEASURED_VALU_INSTS else None),
+                     "limiter": "vector ALU + fp32 matrix instructions (softmax, epilogues, quantisers); the int8 products are hidden under them",
                      # the kernel's second resource: every position streams the packed weights out of the
                      # cache hierarchy (bytes_per_launch / kernel_ms = achieved); `stream_ceiling_TBps` is
                      # what the same number of workgroups reach streaming a buffer of the network's size
@@ -187,7 +190,7 @@ def main() -> int:
                                        "l1_fill_nominal_TBps": 256 * 64 * 2.4e9 / 1e12}},
     }
     from brokefish_amd.hip_impl import stream_rate
-    line["roofline"]["weight_stream"]["stream_ceiling_TBps"] = stream_rate(6_389_760 if kname == "quad" else weight_bytes // a.batch, workgroups=min(a.batch, 4096),
+    line["roofline"]["weight_stream"]["stream_ceiling_TBps"] = stream_rate(6_389_760 if kname == "quad" else 50_626_560 if stress else 6_455_296, workgroups=min(a.batch, 4096),
                                                                            reps=1 if stress else 3)
     # the matrix pipe's measured ceiling for the instruction the kernel uses (register-resident
     # MFMA chains, no memory traffic), next to the datasheet peak that `frac` is quoted against
@@ -199,29 +202,38 @@ def main() -> int:
                           "share_of_total": {k: round(v / ph["total"], 4) for k, v in ph.items() if k != "total"}}
     del model, bd, cd, rd, md
     if headline and not a.no_extras:
-        # configuration 3: the batch sweep (small-batch latency regime), same net, same generator
-        pts = []
-        for nb in (64, 256, 1024, 4096, 16384, 65536):
-            ms, kn, mdl = time_config(net, "int8", nb, iters=20 if nb <= 16384 else 8)
-            pts.append({"batch": nb, "ms_per_launch": ms, "evals_per_s": nb / ms * 1e3, "kernel": kn,
-                        "frac_int8_peak": OPS_PER_EVAL * nb / (ms * 1e-3) / PEAK_INT8_OPS})
-            del mdl
-        line["sweep"] = pts
-        # configuration 4: e4m3 at batch 4096 (products on the fp16 matrix instruction: quoted against both peaks)
-        ms, kn, mdl = time_config(net, "e4m3", 4096)
-        tops = OPS_PER_EVAL * 4096 / (ms * 1e-3)
-        line["e4m3"] = {"batch": 4096, "kernel": kn, "kernel_ms": ms, "evals_per_s": 4096 / ms * 1e3, "achieved_TFLOPs": tops / 1e12,
-                        "frac_fp16_peak_2.5PF": tops / PEAK_FP16_OPS, "frac_fp8_peak_5.0PF": tops / 5.0e15,
-                        "measured_mfma_rate": mfma_rate("e4m3")}
-        del mdl
-        # configuration 5: the 16-layer 512-wide network at batch 16384
+        # configurations 3, 4 and 5 timed in interleaved rounds (every point once per round, median over the
+        # rounds), as the reference's bench does for its variants (bench/bench_model.py:167-193): the batch
+        # sweep (small-batch latency regime; same net, same generator), e4m3 at batch 4096 (products on the
+        # fp16 matrix instruction: quoted against both peaks), the 16-layer 512-wide network at batch 16384
         torch.manual_seed(0)
         wide = BrokefishNet(d_model=512, n_heads=16, d_ff=2048, n_layers=16).eval()
-        ms, kn, mdl = time_config(wide, "int8", 16384, iters=5, warmup=2)
-        line["stress"] = {"batch": 16384, "kernel": kn, "kernel_ms": ms, "evals_per_s": 16384 / ms * 1e3,
+        hip = encoder_impl("hip")
+        mdl8, mdlf, mdlw = hip(net, int8=True, kernel=a.kernel), hip(net, fp8=True, kernel=a.kernel), hip(wide, int8=True)
+        points = [("sweep", nb, mdl8, 20 if nb <= 16384 else 6) for nb in (64, 256, 1024, 4096, 16384, 65536)]
+        points += [("e4m3", 4096, mdlf, 20), ("stress", 16384, mdlw, 4)]
+        inputs = {nb: [t.cuda() for t in positions.random_positions(nb, plies=120, seed=0)] for nb in {p[1] for p in points}}
+        rounds = 3
+        times = {(p[0], p[1]): [] for p in points}
+        for _ in range(rounds):
+            for name, nb, mdl, iters in points:
+                times[(name, nb)].append(mdl.time_kernel_ms(*inputs[nb], warmup=2, iters=iters))
+        med = {k: sorted(v)[len(v) // 2] for k, v in times.items()}
+        line["sweep"] = [{"batch": nb, "ms_per_launch": med[("sweep", nb)], "evals_per_s": nb / med[("sweep", nb)] * 1e3,
+                          "kernel": mdl8.kernel_choice(nb), "frac_int8_peak": OPS_PER_EVAL * nb / (med[("sweep", nb)] * 1e-3) / PEAK_INT8_OPS,
+                          "ms_min_max": [min(times[("sweep", nb)]), max(times[("sweep", nb)])]}
+                         for nb in (64, 256, 1024, 4096, 16384, 65536)]
+        line["timing_protocol"] = f"{rounds} interleaved rounds over the sweep, e4m3 and stress points, median; HIP events on the launch stream"
+        ms = med[("e4m3", 4096)]
+        tops = OPS_PER_EVAL * 4096 / (ms * 1e-3)
+        line["e4m3"] = {"batch": 4096, "kernel": mdlf.kernel_choice(4096), "kernel_ms": ms, "evals_per_s": 4096 / ms * 1e3, "achieved_TFLOPs": tops / 1e12,
+                        "frac_fp16_peak_2.5PF": tops / PEAK_FP16_OPS, "frac_fp8_peak_5.0PF": tops / 5.0e15,
+                        "measured_mfma_rate": mfma_rate("e4m3")}
+        ms = med[("stress", 16384)]
+        line["stress"] = {"batch": 16384, "kernel": mdlw.kernel_choice(16384), "kernel_ms": ms, "evals_per_s": 16384 / ms * 1e3,
                           "achieved_TOPs": OPS_PER_EVAL_STRESS * 16384 / (ms * 1e-3) / 1e12,
                           "frac_int8_peak": OPS_PER_EVAL_STRESS * 16384 / (ms * 1e-3) / PEAK_INT8_OPS}
-        del mdl, wide
+        del mdl8, mdlf, mdlw, wide, inputs
         line["parity"] = parity_report(net)
     if not a.no_cpu:
         cores = physical_cores()

@@ -65,6 +65,9 @@ def build_hip(verbose: bool = False, extra=()) -> str:
     """Compile every translation unit (in parallel: the kernel variants take minutes each)
     and link them into libbrokefish_hip.so."""
     from concurrent.futures import ThreadPoolExecutor
+    # the kernels' timing experiments give wrong results by construction: never in the library
+    if any("BF_EXP_" in f or "BF_TIMING_BUILD" in f for f in list(extra) + HIPCC_FLAGS):
+        raise ValueError("BF_EXP_* / BF_TIMING_BUILD switches are timing experiments and must not be built into the library")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
 

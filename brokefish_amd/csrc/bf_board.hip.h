@@ -66,6 +66,14 @@
 #define BF_OCTO_SETS 4
 #endif
 
+// Timing experiments (BF_EXP_*): compile-time switches that replace a part of a kernel by a
+// cheaper stand-in to measure what that part costs.  Their results are wrong by construction, so
+// they compile only together with BF_TIMING_BUILD, which the library's own build never defines
+// (brokefish_amd/_build.py refuses both).
+#if (defined(BF_EXP_NOF32) || defined(BF_EXP_NOMFMA) || defined(BF_EXP_SAMEBLOCK) || defined(BF_EXP_NOLOAD) || \
+     defined(BF_EXP_HALFLOAD) || defined(BF_EXP_NOBARRIER)) && !defined(BF_TIMING_BUILD)
+#error "BF_EXP_* switches give wrong results: they need BF_TIMING_BUILD and never go into the library"
+#endif
 #ifdef BF_EXP_NOF32   // timing experiment: one vector instruction in place of an fp32 matrix step
 #define BF_F32MMA(a_, b_, c_) ([&]() { v16f r_ = (c_); r_[0] = __builtin_fmaf((a_), (b_), r_[0]); return r_; }())
 #else

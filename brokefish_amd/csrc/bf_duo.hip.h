@@ -14,7 +14,8 @@
 //
 // LDS map (bytes): [xch: 3 slots x 2 positions x 8 waves x 64 floats] [hid: the quantised hidden
 // row, 32 KiB per position] [act: the quantised row of the width, 8 KiB per position] [par: one
-// copy of each quarter's side parameters, shared by its two wavefronts and both positions].
+// copy of each quarter's side parameters, shared by its two wavefronts and both positions]
+// [tok: the activation scale of every token of the row that feeds QKV, per position].
 // During the heads the normalised stream of a position (32 KiB, fp32) overlays its hidden row.
 #pragma once
 
@@ -47,7 +48,8 @@ struct Cfg : Layout<256> {
     static constexpr int ACT_P = NT * FRAG;               // a position's row of the width
     static constexpr int PAR_OFF = ACT_OFF + NP * ACT_P;
     static constexpr int PWL_FLOATS = A_FLOATS + B_FLOATS;
-    static constexpr int LDS_BYTES = PAR_OFF + 4 * PWL_FLOATS * 4;
+    static constexpr int TOK_OFF = PAR_OFF + 4 * PWL_FLOATS * 4;   // activation scale of every token, per position
+    static constexpr int LDS_BYTES = TOK_OFF + NP * 32 * 4;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget: one workgroup per compute unit");
     static_assert(NT * 4 * FRAG <= HID_P, "normalised stream overlay");
 };
@@ -126,13 +128,18 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             lds_barrier();
             t_sync += __builtin_readcyclecounter() - t0_;
         } else {
+#ifdef BF_EXP_NOBARRIER   // timing experiment: no workgroup barriers (results are wrong)
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#else
             lds_barrier();
+#endif
         }
     };
 
     float* const xch = reinterpret_cast<float*>(lds + C::XCH_OFF);
     uint8_t* const hid = lds + C::HID_OFF;
     uint8_t* const act = lds + C::ACT_OFF;
+    float* const tok = reinterpret_cast<float*>(lds + C::TOK_OFF);
     const bool par_owner = sub == 0;
     float* const pA = reinterpret_cast<float*>(lds + C::PAR_OFF) + q * C::PWL_FLOATS;
     float* const pB = pA + C::A_FLOATS;
@@ -218,7 +225,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
     };
     // signed quantiser of both positions' rows: one scale per row; this wave's bytes go to the
     // position's activation buffer, from which every wave reads its B operands
-    auto quant_exchange2 = [&](const float (&y)[NP][16], float (&sa)[NP], int8_t* tap, const size_t (&tap_row)[NP]) {
+    auto quant_exchange2 = [&](const float (&y)[NP][16], float (&sa)[NP], int8_t* tap, const size_t (&tap_row)[NP], bool publish_scales) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
             float am = 0.0f;
@@ -234,6 +241,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             for (int w = 0; w < C::NW; w++) m = __builtin_fmaxf(m, xch[2 * XS + p * PS + w * 64 + lane]);
             m = __builtin_fmaxf(m, partner(m, g));
             sa[p] = m > 0.0f ? (FP8 ? m * 0.125f : div127(m)) : 1.0f;
+            if (publish_scales && wave == 0 && g == 0) tok[p * 32 + t] = sa[p];
             const float inv = 1.0f / sa[p];
             v4i w;
 #pragma unroll
@@ -322,35 +330,43 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         for (int p = 0; p < NP; p++) bl[p] = (size_t)bp[p] * nl_run + li;
         const int lnext = l + 1 < a.l1 ? l + 1 : l;   // after the last layer the same layer is fetched again (and never used)
         const int lbase = li * BPW, lfollow = (lnext - a.l0) * BPW;
-        // Both positions' products with the wave's k-th block of this layer.  Its two halves sit in
-        // register sets 2k % NSETS and (2k + 1) % NSETS; a set is refilled with the wave's half-block
-        // NSETS positions on once it has been consumed.  B0 / B1: fragment 0 of each position's
-        // operand row in LDS (lane offset included).
-#define BF_DUO_WMM(SWAP, k, B0, B1, R, INIT)                                                         \
+        // One position's product with the wave's k-th block of this layer: eight 32-deep steps against
+        // the operand row whose fragment 0 is at BSRC (lane offset included), each fragment fetched
+        // from LDS one step ahead.  The block's two halves sit in register sets 2k % NSETS and
+        // (2k + 1) % NSETS; position 0 goes first and starts the fetch of the half-block NSETS - 1
+        // positions on, position 1 refills the first half's set once it has consumed it.
+        // BETWEEN(s) runs after step s has been issued: an eighth of the previous product's epilogue,
+        // which the vector ALU works through while the matrix pipe runs; nothing is scheduled across
+        // the end of a step.
+#ifndef BF_DUO_AHEAD
+#define BF_DUO_AHEAD 1   // steps between the LDS fetch of an operand fragment and its use
+#endif
+#define BF_DUO_CHAIN(SWAP, k, p, BSRC, INIT, R, BETWEEN)                                             \
     do {                                                                                             \
-        const uint8_t* const b0_ = (B0);                                                             \
-        const uint8_t* const b1_ = (B1);                                                             \
-        (R)[0] = (INIT);                                                                             \
-        (R)[1] = (INIT);                                                                             \
-        fetch_half(2 * (k) + NSETS - 1, lbase, lfollow);                                             \
-        _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++) {                                           \
-            (R)[0] = frag_mma<SWAP>(frt[(2 * (k)) % NSETS][s_], ldsfrag(b0_ + s_ * FRAG), (R)[0]);   \
-            (R)[1] = frag_mma<SWAP>(frt[(2 * (k)) % NSETS][s_], ldsfrag(b1_ + s_ * FRAG), (R)[1]);   \
-        }                                                                                            \
-        fetch_half(2 * (k) + NSETS, lbase, lfollow);                                                 \
-        _Pragma("unroll") for (int s_ = 0; s_ < 4; s_++) {                                           \
-            (R)[0] = frag_mma<SWAP>(frt[(2 * (k) + 1) % NSETS][s_], ldsfrag(b0_ + (4 + s_) * FRAG), (R)[0]); \
-            (R)[1] = frag_mma<SWAP>(frt[(2 * (k) + 1) % NSETS][s_], ldsfrag(b1_ + (4 + s_) * FRAG), (R)[1]); \
+        constexpr int A_ = BF_DUO_AHEAD;                                                             \
+        const uint8_t* const b_ = (BSRC);                                                            \
+        if ((p) == 0) fetch_half(2 * (k) + NSETS - 1, lbase, lfollow);                               \
+        v4i ring_[A_ + 1];                                                                           \
+        _Pragma("unroll") for (int u_ = 0; u_ < A_; u_++) ring_[u_] = ldsfrag(b_ + u_ * FRAG);       \
+        (R) = (INIT);                                                                                \
+        _Pragma("unroll") for (int s_ = 0; s_ < 8; s_++) {                                           \
+            if (s_ + A_ < 8) ring_[(s_ + A_) % (A_ + 1)] = ldsfrag(b_ + (s_ + A_) * FRAG);           \
+            (R) = frag_mma<SWAP>(frt[(2 * (k) + s_ / 4) % NSETS][s_ % 4], ring_[s_ % (A_ + 1)], (R)); \
+            BETWEEN(s_);                                                                             \
+            __builtin_amdgcn_sched_barrier(0);                                                       \
+            if ((p) == 1 && s_ == 3) fetch_half(2 * (k) + NSETS, lbase, lfollow);                    \
         }                                                                                            \
     } while (0)
         const acc_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        auto none = [&](int) {};
+        const uint8_t* const act1 = act0 + C::ACT_P;
 
         // ---- LayerNorm 1, quantise, exchange -----------------------------------------------------------
         float sa[NP];
         {
             float y[NP][16];
             layernorm2(x, pA + C::A_LN1G + 32 * sub, pA + C::A_LN1B + 32 * sub, y);
-            quant_exchange2(y, sa, TAPS ? a.taps.qa_qkv : nullptr, bl);
+            quant_exchange2(y, sa, TAPS ? a.taps.qa_qkv : nullptr, bl, true);
         }
         // the quarter's feed-forward parameters of this layer (the first layer's came with the start)
         if (par_owner && li > 0) {
@@ -366,53 +382,50 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             const float swq = pA[C::A_SW + sub], swk = pA[C::A_SW + TW + sub], swv = pA[C::A_SW + 2 * TW + sub];
             const float bv = pA[C::A_BV + 32 * sub + t];
             acc_t acc[NP];
-            {
-                v4f bq[4];
-                load_tile16(pA + C::A_BQ + 32 * sub, g, bq);
-                BF_DUO_WMM(false, 0, act0, act0 + C::ACT_P, acc, zero);
+            v4f bq[4], bk[4], stok[NP][4];
+            // the epilogues, two accumulator registers at a time (slice s of eight)
+            auto epi_q = [&](int p, int s) {
 #pragma unroll
-                for (int p = 0; p < NP; p++) {
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-#pragma unroll
-                        for (int k = 0; k < 4; k++) qf[p][4 * j + k] = accf(acc[p], 4 * j + k) * sa[p] * swq + bq[j][k];
-                    pin16(qf[p]);
+                for (int e = 2 * s; e < 2 * s + 2; e++) {
+                    qf[p][e] = accf(acc[p], e) * sa[p] * swq + bq[e / 4][e % 4];
                     if (TAPS && a.taps.acc_qkv && live[p])
-#pragma unroll
-                        for (int r = 0; r < 16; r++)
-                            a.taps.acc_qkv[(bl[p] * T + t) * 3 * D + 32 * tile + ch(r, g)] = tapbits<false>(acc[p], r);
+                        a.taps.acc_qkv[(bl[p] * T + t) * 3 * D + 32 * tile + ch(e, g)] = tapbits<false>(acc[p], e);
                 }
-            }
-            {
-                v4f bk[4];
-                load_tile16(pA + C::A_BK + 32 * sub, g, bk);
-                BF_DUO_WMM(false, 1, act0, act0 + C::ACT_P, acc, zero);
+            };
+            auto epi_k = [&](int p, int s) {
 #pragma unroll
-                for (int p = 0; p < NP; p++) {
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-#pragma unroll
-                        for (int k = 0; k < 4; k++) kf[p][4 * j + k] = accf(acc[p], 4 * j + k) * sa[p] * swk + bk[j][k];
-                    pin16(kf[p]);
+                for (int e = 2 * s; e < 2 * s + 2; e++) {
+                    kf[p][e] = accf(acc[p], e) * sa[p] * swk + bk[e / 4][e % 4];
                     if (TAPS && a.taps.acc_qkv && live[p])
-#pragma unroll
-                        for (int r = 0; r < 16; r++)
-                            a.taps.acc_qkv[(bl[p] * T + t) * 3 * D + D + 32 * tile + ch(r, g)] = tapbits<false>(acc[p], r);
+                        a.taps.acc_qkv[(bl[p] * T + t) * 3 * D + D + 32 * tile + ch(e, g)] = tapbits<false>(acc[p], e);
                 }
-            }
-            BF_DUO_WMM(true, 2, act0, act0 + C::ACT_P, acc, zero);
+            };
+            // V tile: rows are tokens, so the activation scale is that of token ch(e, g)
+            auto epi_v = [&](int p, int s) {
 #pragma unroll
-            for (int p = 0; p < NP; p++) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    vf[p][r] = accf(acc[p], r) * __shfl(sa[p], ch(r, g)) * swv + bv;   // V tile: rows are tokens
+                for (int e = 2 * s; e < 2 * s + 2; e++) {
+                    vf[p][e] = accf(acc[p], e) * stok[p][e / 4][e % 4] * swv + bv;
+                    if (TAPS && a.taps.acc_qkv && live[p])
+                        a.taps.acc_qkv[(bl[p] * T + ch(e, g)) * 3 * D + 2 * D + 32 * tile + t] = tapbits<false>(acc[p], e);
                 }
-                pin16(vf[p]);
-                if (TAPS && a.taps.acc_qkv && live[p])
+            };
+            auto eq0 = [&](int s) { epi_q(0, s); };
+            auto eq1 = [&](int s) { epi_q(1, s); };
+            auto ek0 = [&](int s) { epi_k(0, s); };
+            auto ek1 = [&](int s) { epi_k(1, s); };
+            auto ev0 = [&](int s) { epi_v(0, s); };
+            load_tile16(pA + C::A_BQ + 32 * sub, g, bq);
+            BF_DUO_CHAIN(false, 0, 0, act0, zero, acc[0], none);
+            BF_DUO_CHAIN(false, 0, 1, act1, zero, acc[1], eq0);
+            load_tile16(pA + C::A_BK + 32 * sub, g, bk);
+            BF_DUO_CHAIN(false, 1, 0, act0, zero, acc[0], eq1);
+            BF_DUO_CHAIN(false, 1, 1, act1, zero, acc[1], ek0);
+            load_tile16(tok, g, stok[0]);
+            BF_DUO_CHAIN(true, 2, 0, act0, zero, acc[0], ek1);
+            load_tile16(tok + 32, g, stok[1]);
+            BF_DUO_CHAIN(true, 2, 1, act1, zero, acc[1], ev0);
 #pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        a.taps.acc_qkv[(bl[p] * T + ch(r, g)) * 3 * D + 2 * D + 32 * tile + t] = tapbits<false>(acc[p], r);
-            }
+            for (int s = 0; s < 8; s++) epi_v(1, s);
             BF_PHASE(PH_QKV);
 #pragma unroll
             for (int p = 0; p < NP; p++) {
@@ -450,33 +463,32 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         // ---- output projection + residual (this wave's tile) --------------------------------------------
         {
             float so[NP];
-            quant_exchange2(o, so, TAPS ? a.taps.qa_out : nullptr, bl);
+            quant_exchange2(o, so, TAPS ? a.taps.qa_out : nullptr, bl, false);
             acc_t acc[NP];
-            BF_DUO_WMM(false, 3, act0, act0 + C::ACT_P, acc, zero);
             v4f bo[4];
             load_tile16(pA + C::A_BOUT + 32 * sub, g, bo);
             const float sw = pA[C::A_SW + 3 * TW + sub];
+            auto epi_o = [&](int p, int s) {
 #pragma unroll
-            for (int p = 0; p < NP; p++) {
+                for (int e = 2 * s; e < 2 * s + 2; e++) {
+                    x[p][e] = x[p][e] + (accf(acc[p], e) * so[p] * sw + bo[e / 4][e % 4]);
+                    if (TAPS && a.taps.acc_out && live[p])
+                        a.taps.acc_out[(bl[p] * T + t) * D + 32 * tile + ch(e, g)] = tapbits<false>(acc[p], e);
+                }
+            };
+            auto eo0 = [&](int s) { epi_o(0, s); };
+            BF_DUO_CHAIN(false, 3, 0, act0, zero, acc[0], none);
+            BF_DUO_CHAIN(false, 3, 1, act1, zero, acc[1], eo0);
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-#pragma unroll
-                    for (int k = 0; k < 4; k++)
-                        x[p][4 * j + k] = x[p][4 * j + k] + (accf(acc[p], 4 * j + k) * so[p] * sw + bo[j][k]);
-                pin16(x[p]);
-                if (TAPS && a.taps.acc_out && live[p])
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        a.taps.acc_out[(bl[p] * T + t) * D + 32 * tile + ch(r, g)] = tapbits<false>(acc[p], r);
-            }
+            for (int s = 0; s < 8; s++) epi_o(1, s);
         }
-
         BF_PHASE(PH_OUT);
+
         // ---- feed-forward ---------------------------------------------------------------------------------
         {
             float y[NP][16];
             layernorm2(x, pB + C::B_LN2G + 32 * sub, pB + C::B_LN2B + 32 * sub, y);
-            quant_exchange2(y, sa, TAPS ? a.taps.qa_ff1 : nullptr, bl);
+            quant_exchange2(y, sa, TAPS ? a.taps.qa_ff1 : nullptr, bl, false);
         }
         // the attention-phase parameters are dead for both waves of the quarter: fetch the next layer's
         if (par_owner) {
@@ -492,33 +504,38 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         for (int st = 0; st < STEPS; st++) {
             float hf[NP][HT][16];
             float am[NP] = {0.0f, 0.0f};
+            acc_t acc[NP];
+            v4f b1[HT][4];
+            float sw1[HT];
+            auto epi_f = [&](int i, int p, int s) {
 #pragma unroll
-            for (int i = 0; i < HT; i++) {
-                acc_t acc[NP];
-                BF_DUO_WMM(false, 4 + HT * st + i, act0, act0 + C::ACT_P, acc, zero);
-                v4f b1[4];
-                load_tile16(pB + C::B_BFF1 + 128 * st + 32 * (HT * sub + i), g, b1);
-                const float sw = pB[C::B_SW + 4 * st + HT * sub + i];
+                for (int e = 2 * s; e < 2 * s + 2; e++) {
+                    // int8: the ReLU is the saturation of the unsigned quantiser below, and the
+                    // running maximum starts at 0, so negative values need no clamp here
+                    float v = accf(acc[p], e) * sa[p] * sw1[i] + b1[i][e / 4][e % 4];
+                    if constexpr (FP8) v = __builtin_fmaxf(v, 0.0f);
+                    hf[p][i][e] = v;
+                    am[p] = __builtin_fmaxf(am[p], v);
+                    if (TAPS && a.taps.acc_ff1 && live[p])
+                        a.taps.acc_ff1[(bl[p] * T + t) * F + 512 * st + 128 * q + 32 * (HT * sub + i) + ch(e, g)] = tapbits<false>(acc[p], e);
+                }
+            };
+#pragma unroll
+            for (int i = 0; i < HT; i++)
 #pragma unroll
                 for (int p = 0; p < NP; p++) {
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-#pragma unroll
-                        for (int k = 0; k < 4; k++) {
-                            // int8: the ReLU is the saturation of the unsigned quantiser below, and the
-                            // running maximum starts at 0, so negative values need no clamp here
-                            float v = accf(acc[p], 4 * j + k) * sa[p] * sw + b1[j][k];
-                            if constexpr (FP8) v = __builtin_fmaxf(v, 0.0f);
-                            hf[p][i][4 * j + k] = v;
-                            am[p] = __builtin_fmaxf(am[p], v);
-                        }
-                    pin16(hf[p][i]);
-                    if (TAPS && a.taps.acc_ff1 && live[p])
-#pragma unroll
-                        for (int r = 0; r < 16; r++)
-                            a.taps.acc_ff1[(bl[p] * T + t) * F + 512 * st + 128 * q + 32 * (HT * sub + i) + ch(r, g)] = tapbits<false>(acc[p], r);
+                    const int n = NP * i + p;   // product number within the step; the previous one's epilogue runs under it
+                    if (p == 0) {
+                        load_tile16(pB + C::B_BFF1 + 128 * st + 32 * (HT * sub + i), g, b1[i]);
+                        sw1[i] = pB[C::B_SW + 4 * st + HT * sub + i];
+                    }
+                    auto between = [&](int s) {
+                        if (n > 0) epi_f((n - 1) / NP, (n - 1) % NP, s);
+                    };
+                    BF_DUO_CHAIN(false, 4 + HT * st + i, p, act0 + p * C::ACT_P, zero, acc[p], between);
                 }
-            }
+#pragma unroll
+            for (int s = 0; s < 8; s++) epi_f(HT - 1, NP - 1, s);
             // the maxima of consecutive steps go through different exchange slots
             const int xs = (st & 1) ? 0 : 2 * XS;
 #pragma unroll
@@ -562,45 +579,48 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         {
             double o64[NP][16];
             float o32[NP][16];
+            acc_t acc[NP];
+            acc_t init = zero;
+            float sw2[KCF];   // e4m3: one weight scale per k-chunk
+            if constexpr (FP8)
 #pragma unroll
-            for (int cc = 0; cc < KCF; cc++) {
-                acc_t init = zero;
-                if constexpr (!FP8) {
-                    v4i w0[4];
-                    load_tile16i(pB + C::B_WSUM + cc * CW + 32 * sub, g, w0);
+                for (int cc = 0; cc < KCF; cc++) sw2[cc] = pB[C::B_SW + 16 + sub * KCF + cc];
+            auto epi_2 = [&](int cc, int p, int s) {
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
-#pragma unroll
-                        for (int k = 0; k < 4; k++) init[4 * j + k] = w0[j][k];
-                }
-                acc_t acc[NP];
-                BF_DUO_WMM(false, 4 + HT * STEPS + cc, hid0 + 8 * cc * FRAG, hid0 + C::HID_P + 8 * cc * FRAG, acc, init);
-#pragma unroll
-                for (int p = 0; p < NP; p++) {
+                for (int e = 2 * s; e < 2 * s + 2; e++) {
                     if constexpr (FP8) {
-                        const float sw = pB[C::B_SW + 16 + sub * KCF + cc];
-#pragma unroll
-                        for (int r = 0; r < 16; r++) {
-                            const float part = (accf(acc[p], r) * sh[p][cc]) * sw;
-                            o32[p][r] = cc == 0 ? part : o32[p][r] + part;
-                            if (TAPS && a.taps.acc_ff2 && live[p])
-                                a.taps.acc_ff2[((bl[p] * KCF + cc) * T + t) * D + 32 * tile + ch(r, g)] = accbits(acc[p], r);
-                        }
-                        pin16(o32[p]);
+                        const float part = (accf(acc[p], e) * sh[p][cc]) * sw2[cc];
+                        o32[p][e] = cc == 0 ? part : o32[p][e] + part;
                     } else {
                         const double sc = (double)sh[p][cc];
-#pragma unroll
-                        for (int r = 0; r < 16; r++) {
-                            const int full = accbits(acc[p], r);
-                            o64[p][r] = cc == 0 ? (double)full * sc : __builtin_fma((double)full, sc, o64[p][r]);
-                            if (TAPS && a.taps.acc_ff2 && live[p])
-                                a.taps.acc_ff2[((bl[p] * KCF + cc) * T + t) * D + 32 * tile + ch(r, g)] = full;
-                        }
-#pragma unroll
-                        for (int r = 0; r < 16; r++) pin(o64[p][r]);
+                        const int full = accbits(acc[p], e);
+                        o64[p][e] = cc == 0 ? (double)full * sc : __builtin_fma((double)full, sc, o64[p][e]);
                     }
+                    if (TAPS && a.taps.acc_ff2 && live[p])
+                        a.taps.acc_ff2[((bl[p] * KCF + cc) * T + t) * D + 32 * tile + ch(e, g)] = accbits(acc[p], e);
                 }
-            }
+            };
+#pragma unroll
+            for (int cc = 0; cc < KCF; cc++)
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    const int n = NP * cc + p;
+                    if constexpr (!FP8)
+                        if (p == 0) {
+                            v4i w0[4];
+                            load_tile16i(pB + C::B_WSUM + cc * CW + 32 * sub, g, w0);
+#pragma unroll
+                            for (int j = 0; j < 4; j++)
+#pragma unroll
+                                for (int k = 0; k < 4; k++) init[4 * j + k] = w0[j][k];
+                        }
+                    auto between = [&](int s) {
+                        if (n > 0) epi_2((n - 1) / NP, (n - 1) % NP, s);
+                    };
+                    BF_DUO_CHAIN(false, 4 + HT * STEPS + cc, p, hid0 + p * C::HID_P + 8 * cc * FRAG, init, acc[p], between);
+                }
+#pragma unroll
+            for (int s = 0; s < 8; s++) epi_2(KCF - 1, NP - 1, s);
             v4f b2[4];
             load_tile16(pB + C::B_BFF2 + 32 * sub, g, b2);
             const float sw = pB[C::B_SW + 16 + sub];
@@ -619,7 +639,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             }
         }
         BF_PHASE(PH_FF2);
-#undef BF_DUO_WMM
+#undef BF_DUO_CHAIN
         if (TAPS && a.taps.resid)
 #pragma unroll
             for (int p = 0; p < NP; p++)

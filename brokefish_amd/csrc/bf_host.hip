@@ -32,8 +32,9 @@ static bool shape512(const bf_shape* s) {
 static bool board_shape_ok(const bf_shape* s) { return shape_ok(s) || shape512(s); }
 
 // AUTO runs one workgroup of eight wavefronts per compute unit (lowest latency per position) up
-// to this many positions, which is one per compute unit of an MI355X; above it, two workgroups
-// of four wavefronts per compute unit (highest throughput; 256-wide network).
+// to this many positions, which is one per compute unit of an MI355X; above it, the forms built
+// for throughput (256-wide network): two positions per workgroup (int8) or two workgroups of
+// four wavefronts per compute unit (e4m3).
 static const int64_t kBoardMaxN = 256;
 
 template <int DM>
@@ -127,7 +128,10 @@ static int choose_kernel(const bf_eval_args* a) {
             return fail(BF_ERR_UNSUPPORTED, "the two-positions-per-workgroup kernel needs the 256-wide network and board_wstream/board_fparams");
         return BF_KERNEL_DUO;
     case BF_KERNEL_AUTO:
-        if (octo_can) return (twin_can && a->n > kBoardMaxN) ? BF_KERNEL_TWIN : BF_KERNEL_OCTO;
+        // above one position per compute unit: two positions per workgroup for int8 (2-4 % faster
+        // than TWIN from 512 positions up and half its L2 traffic), TWIN for e4m3 (whose operand
+        // conversions leave the two-position form short of registers)
+        if (octo_can) return (twin_can && a->n > kBoardMaxN) ? (a->quant == BF_QUANT_INT8 ? BF_KERNEL_DUO : BF_KERNEL_TWIN) : BF_KERNEL_OCTO;
         if (quad_can) return BF_KERNEL_QUAD;
         return fail(BF_ERR_ARGUMENT, shape512(&a->shape)
                         ? "the 512-wide network runs on the one-position-per-workgroup kernel: int8, board_wstream/board_fparams required"

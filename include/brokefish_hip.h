@@ -168,8 +168,8 @@ typedef struct {
      * QUAD: the wavefront runs on, storing nothing) */
     const uint8_t* active;
     int32_t kernel;         /* enum bf_kernel; AUTO with the board blobs: OCTO for
-                             * n <= bf_board_max_n() and for the 512-wide network, TWIN
-                             * above; without the board blobs QUAD */
+                             * n <= bf_board_max_n() and for the 512-wide network, above that
+                             * DUO (int8) or TWIN (e4m3); without the board blobs QUAD */
     /* which tokens the value rows read (reference brokefish/nn/model.py:551-617): the king of the
      * side to move (BF_VALUE_KING, the default), the mean of the final-normed live tokens
      * (BF_VALUE_POOLED), or the final norm of the mean of the live tokens' residual stream
@@ -187,7 +187,7 @@ typedef struct {
     const int32_t* leaf_count;
 } bf_eval_args;
 
-/* Largest n for which AUTO prefers BOARD over TWIN on the 256-wide network. */
+/* Largest n for which AUTO prefers OCTO over DUO / TWIN on the 256-wide network. */
 int64_t bf_board_max_n(void);
 /* The kernel AUTO would run for these arguments (enum bf_kernel), or a negative bf_status. */
 int bf_kernel_choice(const bf_eval_args* args);

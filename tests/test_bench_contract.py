@@ -27,7 +27,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert d["metric"] == "network evals/sec at batch 4096 int8 on 1 MI355X" and d["unit"] == "evals/s"
     assert d["n_gpus"] == 1 and d["steps"] == 5 and d["warmup"] == 2 and d["higher_is_better"] is True
     assert d["dtype"] == "int8" and d["data"] == "synthetic" and d["vs_baseline"] is None and d["scaling"] == "weak"
-    assert set(d["config"]) == {"workload"} and "batch 4096" in d["config"]["workload"] and "kernel twin" in d["config"]["workload"]
+    assert set(d["config"]) == {"workload"} and "batch 4096" in d["config"]["workload"] and "kernel duo" in d["config"]["workload"]
     assert abs(d["value"] - 4096 / (d["ms_per_step"] * 1e-3)) < 1e-6 * d["value"]
     r = d["roofline"]
     assert r["bound"] == "mfma" and r["unit"] == "TOP/s" and r["peak"] == 5000.0
@@ -40,8 +40,10 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert c["kind"] == "port" and c["unit"] == "evals/s" and c["cores"] >= 1 and c["value"] > 0 and "batch 16" in c["sample"]
     assert c["physical_cores"] >= 1 and c["fp32"]["value"] > 0
     # every configuration is in the default line: the sweep, e4m3 and the 512-wide network
-    assert [p["batch"] for p in d["sweep"]] == [64, 256, 1024, 4096, 16384, 65536]
-    assert all(p["ms_per_launch"] > 0 and p["kernel"] in ("octo", "twin") for p in d["sweep"])
+    assert [p["batch"] for p in d["sweep"]] == [64, 256, 1024, 4096, 16384, 65536] and "interleaved" in d["timing_protocol"]
+    assert all(p["ms_min_max"][0] <= p["ms_per_launch"] <= p["ms_min_max"][1] for p in d["sweep"])
+    assert 0.5 < r["valu_floor_ms"] < r["kernel_ms"] and "vector ALU" in r["limiter"]
+    assert all(p["ms_per_launch"] > 0 and p["kernel"] in ("octo", "duo") for p in d["sweep"])
     e = d["e4m3"]
     assert e["batch"] == 4096 and abs(e["frac_fp16_peak_2.5PF"] - 2 * e["frac_fp8_peak_5.0PF"]) < 1e-9 and e["evals_per_s"] > 5e5
     st = d["stress"]
@@ -49,7 +51,7 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     par = d["parity"]
     assert par["bit_exact_vs_c_checker"] is True and par["masked_argmax_equal"] is True
     assert par["prior_space_vs_int8_emulation"]["max_abs"] < 1e-2 and par["prior_space_vs_int8_emulation"]["edge_set_differs"] == 0
-    assert r["weight_stream"]["bytes_per_launch"] == 4096 * 6_455_296
+    assert r["weight_stream"]["bytes_per_launch"] == 2048 * 6_455_296                 # two positions share a copy
     assert r["weight_stream"]["achieved_TBps"] < 1.1 * r["weight_stream"]["stream_ceiling_TBps"] < 1.1 * r["weight_stream"]["l1_fill_nominal_TBps"]
 
 

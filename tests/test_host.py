@@ -89,17 +89,17 @@ def test_kernel_choice_follows_shape_blobs_and_batch_size():
     a.wstream = a.fparams = a.board_wstream = a.board_fparams = 16      # only tested for NULL here
     cut = lib.bf_board_max_n()
     assert cut == 256                                                    # one position per compute unit
-    for n, want in ((1, 4), (cut, 4), (cut + 1, 3), (4096, 3)):          # OCTO up to the cut, TWIN above
+    for n, want in ((1, 4), (cut, 4), (cut + 1, 5), (4096, 5)):          # int8: OCTO up to the cut, DUO above
         a.n = n
         assert lib.bf_kernel_choice(ctypes.byref(a)) == want
-    for forced in (1, 2, 3, 4):
+    for forced in (1, 2, 3, 4, 5):
         a.n, a.kernel = 4096, forced
         assert lib.bf_kernel_choice(ctypes.byref(a)) == forced
-    a.kernel, a.quant = 0, 1                                            # e4m3: the same rule
+    a.kernel, a.quant = 0, 1                                            # e4m3: OCTO up to the cut, TWIN above
     for n, want in ((1, 4), (cut, 4), (cut + 1, 3), (4096, 3)):
         a.n = n
         assert lib.bf_kernel_choice(ctypes.byref(a)) == want
-    for forced in (1, 2, 3, 4):
+    for forced in (1, 2, 3, 4, 5):
         a.kernel = forced
         assert lib.bf_kernel_choice(ctypes.byref(a)) == forced
     a.kernel, a.quant, a.board_wstream = 0, 0, None                     # no board blobs: always quad
@@ -110,7 +110,7 @@ def test_kernel_choice_follows_shape_blobs_and_batch_size():
     for n in (1, 100000):
         a.n = n
         assert lib.bf_kernel_choice(ctypes.byref(a)) == 4
-    for forced, want in ((1, -2), (2, 2), (3, -2), (4, 4)):
+    for forced, want in ((1, -2), (2, 2), (3, -2), (4, 4), (5, -2)):
         a.kernel = forced
         assert lib.bf_kernel_choice(ctypes.byref(a)) == want
     for forced in (0, 2, 4):                                            # ... and in int8 only
@@ -119,6 +119,22 @@ def test_kernel_choice_follows_shape_blobs_and_batch_size():
     a.quant = 0
     a.kernel = 7
     assert lib.bf_kernel_choice(ctypes.byref(a)) == -1
+
+
+def test_timing_experiments_cannot_reach_the_library():
+    """The kernels' BF_EXP_* switches give wrong results by construction: the build refuses them,
+    and the sources refuse to compile them without BF_TIMING_BUILD."""
+    from brokefish_amd import _build
+    assert not any("BF_EXP" in f or "BF_TIMING" in f for f in _build.HIPCC_FLAGS)
+    for extra in (["-DBF_EXP_NOLOAD"], ["-DBF_TIMING_BUILD"]):
+        with pytest.raises(ValueError):
+            _build.build_hip(extra=extra)
+    src = open(os.path.join(_build.CSRC, "bf_board.hip.h")).read()
+    assert '#error "BF_EXP_* switches give wrong results' in src
+    import re
+    used = set(re.findall(r"BF_EXP_[A-Z0-9]+", src + open(os.path.join(_build.CSRC, "bf_duo.hip.h")).read()))
+    guard = src[src.index("#if (defined(BF_EXP_"):src.index("#error")]
+    assert used and all(u in guard for u in used), used
 
 
 def test_board_packing_layout_and_sizes():

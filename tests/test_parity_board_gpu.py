@@ -33,7 +33,7 @@ def _make(d, heads, layers, nv=1, seed=0):
 @pytest.fixture(scope="module")
 def base():
     net, sd = _make(256, 8, 8)
-    return (net, sd, {k: encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=k) for k in ("board", "twin", "octo")},
+    return (net, sd, {k: encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=k) for k in ("board", "twin", "octo", "duo")},
             encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel="quad"), c_oracle.COracle(sd))
 
 
@@ -55,7 +55,7 @@ def _bits_equal(a: torch.Tensor, b: np.ndarray) -> bool:
                                         == b.view(np.int32 if b.dtype == np.float32 else b.dtype)).all())
 
 
-@pytest.mark.parametrize("kernel", ["board", "twin", "octo"])
+@pytest.mark.parametrize("kernel", ["board", "twin", "octo", "duo"])
 def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base, kernel):
     net, sd, boards, quad, co = base
     board = boards[kernel]
@@ -66,7 +66,7 @@ def test_base_network_bit_exact_against_the_c_checker_with_every_tap(base, kerne
         assert _bits_equal(got[k], want[k]), k
 
 
-@pytest.mark.parametrize("kernel", ["board", "twin", "octo"])
+@pytest.mark.parametrize("kernel", ["board", "twin", "octo", "duo"])
 def test_heads_alone_and_a_layer_range_from_a_given_residual_stream(base, kernel):
     # a run of no layers starts the weight stream at the head blocks (no layer block is fetched,
     # none exists to fetch past the last layer); a run of some layers continues into them
@@ -86,7 +86,7 @@ def test_heads_alone_and_a_layer_range_from_a_given_residual_stream(base, kernel
         assert _bits_equal(tail[k], want[k]), k
 
 
-@pytest.mark.parametrize("kernel", ["board", "twin", "octo"])
+@pytest.mark.parametrize("kernel", ["board", "twin", "octo", "duo"])
 @pytest.mark.parametrize("nv", [1, 3])
 def test_the_kernels_return_the_same_bits(base, nv, kernel):
     if nv == 1:
@@ -122,11 +122,11 @@ def test_automatic_choice_switches_kernel_by_batch_size_without_changing_results
     auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
     cut = int(auto._lib.bf_board_max_n())
     assert auto.kernel_choice(1) == "octo" and auto.kernel_choice(cut) == "octo"
-    assert auto.kernel_choice(cut + 1) == "twin" and auto.kernel_choice(4096) == "twin"
+    assert auto.kernel_choice(cut + 1) == "duo" and auto.kernel_choice(4096) == "duo"
     assert "by batch size" in auto.label
     b, c, r, m = positions.random_positions(cut + 4, plies=120, seed=22)
     bd, cd, rd, md = _dev(b, c, r, m)
-    big = [t.clone() for t in auto.forward_masked(bd, cd, rd, md)]                        # two workgroups per CU
+    big = [t.clone() for t in auto.forward_masked(bd, cd, rd, md)]                        # two positions per workgroup
     small = auto.forward_masked(bd[:cut], cd[:cut], rd[:cut], md[:cut])                  # one
     for x, y in zip(big, small):
         assert torch.equal(x[:cut], y)
@@ -156,8 +156,9 @@ def test_e4m3_on_the_throughput_kernel_equals_the_four_per_workgroup_kernel(base
         assert tt[k].dtype == tq[k].dtype and torch.equal(tt[k].view(torch.uint8), tq[k].view(torch.uint8)), k
     int8 = boards["twin"].forward_full(bd, cd, rd)[0]
     assert not torch.equal(int8, twin.forward_full(bd, cd, rd)[0])
-    # the one-workgroup-per-compute-unit kernels carry the format too, and AUTO switches by size
-    for kernel in ("board", "octo"):
+    # the other one-position kernels and the two-position kernel carry the format too, and AUTO
+    # switches by size
+    for kernel in ("board", "octo", "duo"):
         other = encoder_impl("hip")(net, fp8=True, out_dtype=torch.float32, kernel=kernel)
         for x, y in zip(other.forward_masked(bd, cd, rd, md), got):
             assert torch.equal(x, y), kernel
@@ -171,7 +172,7 @@ def test_e4m3_on_the_throughput_kernel_equals_the_four_per_workgroup_kernel(base
         assert torch.equal(x, y[:200])
 
 
-@pytest.mark.parametrize("kernel", ["board", "twin", "octo", "quad"])
+@pytest.mark.parametrize("kernel", ["board", "twin", "octo", "duo", "quad"])
 def test_skipped_positions_keep_their_output_rows(base, kernel):
     # the search's flat leaf staging: only flagged leaves are evaluated (reference
     # brokefish/search/cuda_impl.py:137-145), the others cost nothing and change nothing
@@ -193,7 +194,7 @@ def test_skipped_positions_keep_their_output_rows(base, kernel):
         model.forward_full(bd, cd, rd, md, active=act[:10])
 
 
-@pytest.mark.parametrize("kernel", ["twin", "octo", "board", "quad"])
+@pytest.mark.parametrize("kernel", ["twin", "octo", "duo", "board", "quad"])
 def test_compacted_leaf_list_with_a_device_side_count_equals_the_flag_route(base, kernel):
     # the "compacted list plus a count" of the reference's design retrospective
     # (docs/journal/2026-08-09-kernel-design-retrospective.md:140-154) over its flat leaf staging
@@ -241,7 +242,7 @@ def test_compacted_leaf_list_with_a_device_side_count_equals_the_flag_route(base
 def test_full_batch_at_4096_on_the_throughput_kernel(base):
     net, sd, boards, quad, co = base
     auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)
-    assert auto.kernel_choice(4096) == "twin"
+    assert auto.kernel_choice(4096) == "duo"
     b, c, r, m = positions.random_positions(4096, plies=120, seed=0)
     bd, cd, rd, md = _dev(b, c, r, m)
     p, q, v, best = [t.clone() for t in auto.forward_masked(bd, cd, rd, md)]
@@ -266,7 +267,7 @@ def test_largest_batch_of_the_sweep_is_independent_of_batch_composition(base):
     small = [t.clone() for t in model.forward_masked(*_dev(b, c, r, m))]
     g = torch.Generator().manual_seed(7)
     order = torch.cat([torch.randperm(2048, generator=g) for _ in range(32)])
-    assert model.kernel_choice(65536) == "twin"
+    assert model.kernel_choice(65536) == "duo"
     big = model.forward_masked(*_dev(b[order], c[order], r[order], m[order]))
     od = order.cuda()
     for got, want in zip(big, small):
@@ -356,7 +357,7 @@ def test_pooled_value_heads_bit_exact_on_every_kernel(head, nv):
     assert (c < 0).any() and (c > 0).any()
     want = c_oracle.COracle(sd).forward(b.numpy(), c.numpy(), r.numpy(), mask=m.numpy())
     bd, cd, rd, md = _dev(b, c, r, m)
-    for kernel in ("twin", "octo", "board", "auto"):
+    for kernel in ("twin", "octo", "duo", "board", "auto"):
         model = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=kernel)
         assert model.vmode == {"pooled": 1, "prenorm": 2}[head]
         p, q, v, best = model.forward_masked(bd, cd, rd, md)

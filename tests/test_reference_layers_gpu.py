@@ -24,7 +24,7 @@ from brokefish_amd.net import BrokefishNet
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("kernel", ["twin", "octo", "board", "quad"])
+@pytest.mark.parametrize("kernel", ["twin", "octo", "duo", "board", "quad"])
 def test_one_layer_from_the_references_residual_stream(kernel, capsys):
     fx, net, sd, b, c, r = reflayers.load()
     model = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32, kernel=kernel)

@@ -32,7 +32,7 @@ def test_extension_binding_returns_the_bits_of_the_ctypes_binding_on_the_current
     net = BrokefishNet(n_value=3).eval().randomise_layers_(seed=2)
     b, c, r, m = (t.cuda() for t in positions.random_positions(333, plies=120, seed=9))
     act = (torch.arange(333, device="cuda") % 3 != 0)
-    for kernel in ("auto", "twin", "octo", "board", "quad"):
+    for kernel in ("auto", "twin", "octo", "duo", "board", "quad"):
         for fp8 in (False, True):
             kw = dict(fp8=True) if fp8 else dict(int8=True)
             te = encoder_impl("hip")(net, kernel=kernel, binding="torch", **kw)
