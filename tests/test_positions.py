@@ -99,3 +99,64 @@ def test_mask_agrees_with_movegen_and_step():
     # zero plies is the initial position with its 20 legal moves
     b0, c0, _, m0 = positions.random_positions_np(4, plies=0, seed=1)
     assert (c0 == 1).all() and all(int(np.unpackbits(m0[i].view(np.uint8)).sum()) == 20 for i in range(4))
+
+
+# --------------------------------------------------------------------------- #
+# The reference's own edge-case positions (tests/edge_positions.py), against what the rules of
+# chess fix for them.  The device twin of this test is tests/test_edge_positions_gpu.py.
+# --------------------------------------------------------------------------- #
+
+def _edge_masks():
+    import edge_positions as ep
+    boards, control = ep.boards_of()
+    mask, check = positions.movegen(boards, control)
+    by = {n: i for i, n in enumerate(ep.NAMES)}
+    return ep, boards, control, mask, check, by
+
+
+def check_edge_position_facts(ep, boards, control, mask, check, by):
+    """Facts chess fixes for the edge-case positions, given any generator's masks."""
+    sq = ep.square
+    count = lambda n: sum(bin(int(w)).count("1") for w in mask[by[n]])
+    mv = lambda n: ep.moves_of(boards[by[n]], mask[by[n]])
+    assert count("max-mobility") == 218 and count("startpos") == 20
+    # nine white queens: one in the queen's slot, eight living in pawn slots
+    b = boards[by["max-mobility"]]
+    assert sum(1 for w in b[:16] if not w & 0x800 and (w >> 6) & 7 == 4) == 9
+    assert sum(1 for w in b[:8] if not w & 0x800 and (w >> 6) & 7 == 4) == 8
+    assert int(((boards[by["bare-kings-and-a-rook"]] & 0x800) == 0).sum()) == 3
+    # mate (the fool's mate: in check, no move) and stalemate (not in check, no move): all-zero masks
+    assert check[by["check-by-queen"]] and not mask[by["check-by-queen"]].any()
+    assert not check[by["stalemate-queen"]] and not mask[by["stalemate-queen"]].any()
+    assert mv("single-reply-rook") == {(sq("g8"), sq("h8"))}
+    assert not check[by["white-queen-on-h4-black-to-move"]] and count("white-queen-on-h4-black-to-move") == 25
+    # castling: both ways when free, none out of check, without rights or through a piece
+    e1, e8 = sq("e1"), sq("e8")
+    assert {(e1, sq("g1")), (e1, sq("c1"))} <= mv("castle-both-white")
+    assert {(e8, sq("g8")), (e8, sq("c8"))} <= mv("castle-both-black")
+    for n, k, tg in (("castle-white-in-check", e1, ("g1", "c1")), ("castle-black-in-check", e8, ("g8", "c8")),
+                     ("castle-rights-lost", e1, ("g1", "c1"))):
+        assert not {(k, sq(t)) for t in tg} & mv(n), n
+    assert check[by["castle-white-in-check"]] and check[by["castle-black-in-check"]]
+    blocked = mv("castle-blocked")
+    assert (e1, sq("c1")) in blocked and (e1, sq("g1")) not in blocked       # the knight stands on g1
+    # en passant: taken when it is legal (also as the answer to the pawn's check, and by either
+    # neighbour), absent when it would open the rank between queen and king
+    assert (sq("d4"), sq("e3")) in mv("en-passant-plain")
+    assert {(sq("d4"), sq("e3")), (sq("f4"), sq("e3"))} <= mv("en-passant-two-capturers")
+    assert (sq("d4"), sq("e3")) not in mv("en-passant-pinned") and (sq("d4"), sq("d3")) in mv("en-passant-pinned")
+    assert check[by["en-passant-out-of-check"]] and (sq("e4"), sq("d3")) in mv("en-passant-out-of-check")
+    # promotions by push and by capture; the pinned pawn may not move; checks restrict the replies
+    assert (sq("a7"), sq("a8")) in mv("promotion-by-push")
+    assert not any(f == sq("d2") for f, _ in mv("pinned-pawn"))
+    assert check[by["check-by-bishop"]] and 0 < count("check-by-bishop") < 10
+    assert check[by["promotion-race"]] and count("promotion-race") == 2             # the b2 pawn gives check
+    # the fifty-move clock is carried in the control word: magnitude = clock + 1
+    assert control[by["fifty-move-100"]] == 101 and control[by["fifty-move-99"]] == 100
+    # four legal replies, each the only bit of its word and each bit 62: the words sum to 2**64
+    words = [int(w) for w in mask[by["mask-words-sum-to-2-pow-64"]] if w]
+    assert words == [1 << 62] * 4 and sum(words) == 1 << 64
+
+
+def test_reference_edge_case_positions_on_the_cpu_generator():
+    check_edge_position_facts(*_edge_masks())
