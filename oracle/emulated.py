@@ -309,7 +309,7 @@ def forward(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8
 
 
 def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mode: str = "int8",
-                          n_heads: Optional[int] = None, eps: float = 1e-5):
+                          n_heads: Optional[int] = None, eps: float = 1e-5, taps: Optional[dict] = None):
     """The same forward, but with the encoder stack run by torch's own
     ``nn.TransformerEncoder`` / ``nn.MultiheadAttention`` modules, exactly the modules the
     reference model is built from (brokefish/nn/model.py:303-311).
@@ -320,7 +320,9 @@ def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mod
     output projections), with the attention fast path switched off so the module really
     calls ``F.linear``; ``linear2`` gets the unsigned quantiser.  Under the torch version
     that wrote ``tests/golden/reference_vectors.npz`` this reproduces the reference's
-    emulated forward bit for bit, which is what pins the composition.
+    emulated forward bit for bit, which is what pins the composition.  ``taps`` (int8 mode)
+    collects, per layer, the operand bytes, accumulators and float64 quotients of the four
+    diverted matmuls under the names ``forward`` uses (``qa_qkv`` ... ``quot_ff2``).
     """
     from torch import nn
 
@@ -333,12 +335,14 @@ def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mod
                                        norm_first=True, dropout=0.0, layer_norm_eps=eps)
     stack = nn.TransformerEncoder(layer, num_layers=n_layers, norm=None, enable_nested_tensor=False).eval()
     stack.load_state_dict({k[len("encoder."):]: v for k, v in sd.items() if k.startswith("encoder.")})
-    unsigned_of = {}
+    unsigned_of, name_of = {}, {}
     for lay in stack.layers:
         unsigned_of[id(lay.self_attn.in_proj_weight)] = False
         unsigned_of[id(lay.self_attn.out_proj.weight)] = False
         unsigned_of[id(lay.linear1.weight)] = False
         unsigned_of[id(lay.linear2.weight)] = True
+        name_of.update({id(lay.self_attn.in_proj_weight): "qkv", id(lay.self_attn.out_proj.weight): "out",
+                        id(lay.linear1.weight): "ff1", id(lay.linear2.weight): "ff2"})
     plain_linear = F.linear
     hits = [0]
 
@@ -349,7 +353,7 @@ def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mod
         hits[0] += 1
         if mode == "e4m3":
             return fp8_linear(inp, weight, bias)
-        return int8_linear(inp, weight, bias, unsigned=u)
+        return int8_linear(inp, weight, bias, unsigned=u, taps=taps, name=name_of[id(weight)])
 
     fast = torch.backends.mha.get_fastpath_enabled()
     if mode != "fp32":
@@ -363,6 +367,14 @@ def forward_library_stack(sd: Dict[str, torch.Tensor], boards, control, rep, mod
         torch.backends.mha.set_fastpath_enabled(fast)
     if mode != "fp32" and hits[0] != 4 * n_layers:
         raise AssertionError(f"{hits[0]} matmuls were diverted, expected {4 * n_layers}")
+    if taps:
+        # torch's attention module runs its two projections on [token, board, channel]; bring
+        # their rows into the [board, token] order of everything else
+        n, t = x.shape[0], x.shape[1]
+        for name in ("qkv", "out"):
+            for key in ("qa_", "quot_"):
+                taps[key + name] = [v.view(t, n, -1).transpose(0, 1).reshape(n * t, -1) for v in taps[key + name]]
+            taps["acc_" + name] = [v.view(v.shape[0], t, n, -1).transpose(1, 2).reshape(v.shape[0], n * t, -1) for v in taps["acc_" + name]]
     h_raw = h
     h = F.layer_norm(h_raw, (d,), sd["norm_f.weight"], sd["norm_f.bias"], eps)
     policy = plain_linear(h, sd["policy.weight"])
