@@ -5,7 +5,11 @@ the evaluator's outputs (docs/reference/search.md:616-636, steps 2-6; the torch 
 brokefish/search/torch_impl.py:962-1033 with `_promotion_targets` at :948-960).  Only ``tests/``
 imports this module.
 
-Pins (tests/test_expand.py): the canonical order and the four-way promotion fan-out on hand-built
+Pins (tests/test_expand.py): what the reference's own ``Search._expand`` wrote for 38 positions
+(the eight golden positions and the reference's edge-case positions, 218 candidates among them) at
+E = 96 and E = 16 with formula logits (tests/golden/reference_vectors_expand.npz, written by
+``tests/golden/make_golden.py expand``): move codes, edge and candidate counts exactly, priors to
+fp16 rounding, truncated mass to 2e-6; the canonical order and the four-way promotion fan-out on hand-built
 positions, the properties the reference's own tests assert (tests/test_search.py:317-372: order
 sorted by (move, type), edges = mask bits + 3 per promoting move, priors sum to 1, nothing beyond
 n_edges, the four edges of a promoting move split its mass by softmax(promo), truncation keeps

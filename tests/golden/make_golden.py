@@ -36,6 +36,14 @@ What it records, and why these need the reference itself rather than a closed fo
   value of the pooled / prenorm value heads (model.py:576-617), 1 and 3 value rows, in fp32 and
   int8-simulated, on the eight positions.
 
+* (fourth file, ``python tests/golden/make_golden.py expand``, reference_vectors_expand.npz) the
+  search's expand step as the reference's own ``Search._expand`` performs it
+  (brokefish/search/torch_impl.py:962-1033) at E = 96 and E = 16 on the eight positions above and
+  the reference's edge-case positions (tests/edge_positions.py), with formula logits: edge moves,
+  fp16 priors, edge counts, node values, candidate counts and the truncated prior mass; and on the
+  way the position words of ``env.from_fen`` and the legal-move words and check flags of
+  ``env.movegen`` (brokefish/env/torch_impl.py:781, :254) for the edge-case positions.
+
 Inputs are regenerated from the formulas below by the tests; only outputs are stored.
 """
 from __future__ import annotations
@@ -285,5 +293,51 @@ def main_layers() -> int:
     return 0
 
 
+def expand_logits(n: int):
+    """Formula logits for the expand vectors: policy [n,32,64], promo [n,32,4], value [n] in (-1, 1)."""
+    policy = formula((n, 32, 64), 7907, 13, 4001, 0.0015)
+    promo = formula((n, 32, 4), 6101, 5, 811, 0.004)
+    value = formula((n,), 397, 3, 199, 0.0099)
+    return policy, promo, value
+
+
+def main_expand() -> int:
+    sys.path.insert(0, REFERENCE)
+    sys.path.insert(0, os.path.dirname(HERE))                       # tests/: the list of edge-case FENs
+    sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))      # the repository root
+    from brokefish.env import torch_impl as env
+    from brokefish.search.torch_impl import Search, SearchConfig
+    import edge_positions as ep
+
+    fb, fc = zip(*(env.from_fen(f) for _, f in ep.ALL))
+    fen_boards, fen_control = torch.cat(fb), torch.cat(fc)
+    gb, gc, _ = positions()
+    boards = torch.cat([gb, fen_boards.to(torch.int16)])
+    control = torch.cat([gc, fen_control.to(torch.int16)])
+    n = boards.shape[0]
+    mask, in_check = env.movegen(boards, control)
+    policy, promo, value = expand_logits(n)
+    out = {"fen_boards": fen_boards.to(torch.int16).numpy(), "fen_control": fen_control.to(torch.int16).numpy(),
+           "mask": mask.numpy(), "in_check": in_check.numpy()}
+    for E in (96, 16):
+        s = Search(SearchConfig(n=1, B=n, E=E), evaluate=None, device="cpu", check_invariants=False)
+        s.node_board[:, 0] = boards
+        s.node_control[:, 0] = control
+        rec = {}
+        s.stats.on_expand = lambda count, n_edges, dropped, do: rec.update(count=count.clone(), dropped=dropped.clone())
+        s._expand(torch.zeros(n, dtype=torch.long), mask, torch.ones(n, dtype=torch.bool), policy, promo, value)
+        out[f"edge_move_E{E}"] = s.edge_move[:, 0].numpy().copy()
+        out[f"edge_prior_E{E}"] = s.edge_prior[:, 0].numpy().copy()
+        out[f"n_edges_E{E}"] = s.node_nedges[:, 0].numpy().copy()
+        out[f"node_value_E{E}"] = s.node_value[:, 0].numpy().copy()
+        out[f"count_E{E}"] = rec["count"].numpy().astype(np.int32)
+        out[f"dropped_E{E}"] = rec["dropped"].numpy().astype(np.float32)
+    path = os.path.join(HERE, "reference_vectors_expand.npz")
+    np.savez_compressed(path, **out)
+    print(f"wrote {path}: {os.path.getsize(path)} bytes, {n} positions, counts {out['count_E96'].tolist()}")
+    return 0
+
+
 if __name__ == "__main__":
-    raise SystemExit(main_layers() if sys.argv[1:] == ["layers"] else main())
+    mode = sys.argv[1:]
+    raise SystemExit(main_layers() if mode == ["layers"] else main_expand() if mode == ["expand"] else main())

@@ -1,7 +1,9 @@
 """The search's expand step behind the evaluator (docs/reference/search.md:616-636).
 
-CPU part: pins ``oracle/expand.py`` by hand-built positions, by the properties the reference's
-own tests assert (tests/test_search.py:317-372) and by brute-force definitions on small cases.
+CPU part: pins ``oracle/expand.py`` by what the reference's own ``Search._expand`` wrote for 38
+positions (tests/golden/reference_vectors_expand.npz), by hand-built positions, by the properties
+the reference's own tests assert (tests/test_search.py:317-372) and by brute-force definitions on
+small cases.
 GPU part (marked): the HIP kernel against that checker through the C-ABI -- move codes, edge
 counts and candidate counts exactly; priors to fp16 rounding of the exact value (tolerance
 6e-4 relative + 6e-8: half an fp16 ulp plus the fp32 evaluation error); the kept set under
@@ -117,6 +119,66 @@ def test_truncation_keeps_the_largest_with_ties_by_order_brute_force():
 
 
 # --------------------------------------------------------------------------- #
+# What the reference's own Search._expand wrote (tests/golden/reference_vectors_expand.npz, made by
+# `python tests/golden/make_golden.py expand`: brokefish/search/torch_impl.py:962-1033 run on the
+# eight golden positions and the reference's edge-case positions with formula logits, E = 96 and 16)
+# --------------------------------------------------------------------------- #
+
+def _reference_expand_case():
+    import os
+    import sys
+    here = os.path.dirname(os.path.abspath(__file__))
+    sys.path.insert(0, os.path.join(here, "golden"))
+    import make_golden as mg
+    import edge_positions as ep
+    g = np.load(os.path.join(here, "golden", "reference_vectors_expand.npz"))
+    gb, gc, _ = mg.positions()
+    fb, fc = ep.boards_of()
+    boards = np.concatenate([gb.numpy().view(np.uint16), fb])
+    control = np.concatenate([gc.numpy(), fc])
+    pol, pro, val = [t.numpy() for t in mg.expand_logits(boards.shape[0])]
+    return g, boards, control, pol, pro, val, ep
+
+
+def _well_formed(boards):
+    """No two live slots on one square (three of the eight hand-built golden positions keep a
+    bishop under the castled rook: fine for the evaluator they were made for, which reads slots,
+    but not a chess position, and generators may differ on them)."""
+    ok = np.ones(boards.shape[0], bool)
+    for i, b in enumerate(boards):
+        sq = [int(w) & 63 for w in b if not int(w) & 0x800]
+        ok[i] = len(sq) == len(set(sq))
+    return ok
+
+
+def test_position_words_and_legal_moves_equal_the_references_on_its_edge_cases():
+    # the reference's own from_fen and movegen (brokefish/env/torch_impl.py:781, :254) on the
+    # same FEN strings and on the eight golden positions
+    g, boards, control, *_ , ep = _reference_expand_case()
+    n_fen = len(ep.ALL)
+    assert (boards[-n_fen:].view(np.int16) == g["fen_boards"]).all() and (control[-n_fen:] == g["fen_control"]).all()
+    mask, check = positions.movegen(boards, control)
+    ok = _well_formed(boards)
+    assert ok.sum() == boards.shape[0] - 3 and ok[-n_fen:].all()
+    assert (mask.view(np.int64)[ok] == g["mask"][ok]).all()
+    assert ((check != 0)[ok] == g["in_check"][ok]).all()
+
+
+@pytest.mark.parametrize("E", [96, 16])
+def test_checker_reproduces_the_references_expand(E):
+    g, boards, control, pol, pro, val, ep = _reference_expand_case()
+    out = ox.expand(pol, pro, val, g["mask"], boards, control, E)
+    assert (out["count"] == g[f"count_E{E}"]).all() and (out["n_edges"] == g[f"n_edges_E{E}"]).all()
+    assert out["count"].max() == 218 and (out["count"] > E).sum() >= (1 if E == 96 else 20)
+    assert (out["edge_move"] == g[f"edge_move_E{E}"]).all()          # no near-tie at the cut in these vectors
+    assert out["margin"].min() > 1e-4
+    ref = g[f"edge_prior_E{E}"].astype(np.float64)                   # fp16 of the reference's fp32 softmax
+    assert (np.abs(out["edge_prior"] - ref) <= 5e-4 * out["edge_prior"] + 6e-8).all()
+    assert np.abs(out["dropped"] - g[f"dropped_E{E}"]).max() < 2e-6
+    assert np.abs(out["node_value"] - g[f"node_value_E{E}"].astype(np.float64)).max() <= 2.5e-4
+
+
+# --------------------------------------------------------------------------- #
 # GPU
 # --------------------------------------------------------------------------- #
 
@@ -226,3 +288,24 @@ def test_forward_expand_runs_the_evaluator_and_the_expansion_back_to_back():
         expand_edges(p, q.float(), v, md, bd, cd, 96)
     with pytest.raises(ValueError):
         expand_edges(p, q, v, md, bd, cd, 300)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("E", [96, 16])
+def test_kernel_reproduces_the_references_expand(E):
+    from brokefish_amd.hip_impl import expand_edges
+    g, boards, control, pol, pro, val, ep = _reference_expand_case()
+    dev = lambda x: torch.from_numpy(np.ascontiguousarray(x)).cuda()
+    got = expand_edges(dev(pol), dev(pro), dev(val), dev(g["mask"]), dev(boards.view(np.int16)), dev(control), E)
+    assert (got["count"].cpu().numpy() == g[f"count_E{E}"]).all() and (got["n_edges"].cpu().numpy() == g[f"n_edges_E{E}"]).all()
+    assert (got["edge_move"].cpu().numpy() == g[f"edge_move_E{E}"]).all()
+    ref = g[f"edge_prior_E{E}"].astype(np.float64)
+    ep16 = got["edge_prior"].float().cpu().numpy().astype(np.float64)
+    assert (np.abs(ep16 - ref) <= 1.2e-3 * ref + 1.2e-7).all()         # both sides are fp16 roundings: one ulp apart at most
+    assert np.abs(got["dropped"].cpu().numpy() - g[f"dropped_E{E}"]).max() < 2e-6
+    assert np.abs(got["node_value"].float().cpu().numpy() - g[f"node_value_E{E}"].astype(np.float32)).max() <= 5e-4
+    # and the device's own move generation gives the reference's masks on these positions
+    from brokefish_amd.hip_impl import movegen
+    m, chk = movegen(dev(boards.view(np.int16)), dev(control))
+    ok = _well_formed(boards)
+    assert (m.cpu().numpy()[ok] == g["mask"][ok]).all() and (chk.cpu().numpy()[ok] == g["in_check"][ok]).all()
