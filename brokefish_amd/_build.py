@@ -83,6 +83,10 @@ def build_hip(verbose: bool = False, extra=()) -> str:
     with ThreadPoolExecutor(max_workers=min(len(HIP_SOURCES), os.cpu_count() or 4)) as pool:
         objs = list(pool.map(compile_one, HIP_SOURCES))
     _run([hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB] + objs)
+    # the extension module is compiled against this library's header: one built earlier may not
+    # match the library any more, so it goes and build_torch_ext() makes the new one
+    if os.path.exists(TORCH_EXT):
+        os.remove(TORCH_EXT)
     return HIP_LIB
 
 

@@ -176,7 +176,7 @@ __device__ __forceinline__ unsigned quant4(float v0, float v1, float v2, float v
     } else {
         // Adding 1.5 * 2^23 rounds to nearest even and leaves the integer in the low bits of the sum;
         // the sub-dword form of the add writes that low byte straight into its place in the packed
-        // dword (checked on the GPU against rint on four million values and the ties).
+        // dword (held against rint on the host, ties included, by tests/test_quantiser_gpu.py).
         const float magic = 12582912.0f;
         unsigned w;
         asm("v_add_f32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(w) : "v"(qf[0]), "v"(magic));
@@ -189,9 +189,9 @@ __device__ __forceinline__ unsigned quant4(float v0, float v1, float v2, float v
 
 // The unsigned int8 quantiser of the feed-forward hidden row with the ReLU folded in: four
 // correctly rounded quotients v / sa, converted with v_cvt_pk_u8_f32 -- round to nearest even,
-// saturating to [0, 255], so a negative input gives 0 exactly as max(v, 0) would (checked on the
-// GPU against rint + clamp on two million values and every tie k + 0.5) -- each conversion
-// writing its own byte of the dword.
+// saturating to [0, 255], so a negative input gives 0 exactly as max(v, 0) would (held against
+// rint + clamp on the host, every tie k + 0.5 included, by tests/test_quantiser_gpu.py) -- each
+// conversion writing its own byte of the dword.
 __device__ __forceinline__ unsigned quant4_relu_u8(float v0, float v1, float v2, float v3, float sa, float inv) {
     const float v[4] = {v0, v1, v2, v3};
     unsigned w = 0;

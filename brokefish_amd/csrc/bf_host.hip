@@ -62,6 +62,8 @@ extern "C" size_t bf_board_fparams_floats(const bf_shape* s) {
 
 extern "C" int64_t bf_board_max_n(void) { return kBoardMaxN; }
 
+extern "C" uint64_t bf_abi_tag(void) { return BF_ABI_TAG; }
+
 extern "C" size_t bf_wstream_bytes(const bf_shape* s) {
     if (!shape_ok(s)) return 0;
     return ((size_t)s->n_layers * bf::LAYER_GROUPS + bf::HEAD_GROUPS) * bf::GROUP;

@@ -158,7 +158,11 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
     if (a.leaf_index) {
         valid = board_raw < a.n && board_raw < *a.leaf_count;
         b = __builtin_amdgcn_readfirstlane(a.leaf_index[valid ? board_raw : 0]);
-        b = (b >= 0 && b < a.n) ? b : 0;        // an idle wave may read an unwritten entry
+        // an entry that is not a position of this launch is skipped like a slot past the count (the
+        // wave stays for the workgroup's barriers and stores nothing); an idle wave may read an
+        // unwritten entry
+        valid = valid && b >= 0 && b < a.n;
+        b = valid ? b : 0;
     } else {
         valid = board_raw < a.n && !(a.active && !a.active[board_raw < a.n ? board_raw : 0]);
         b = valid ? board_raw : a.n - 1;        // idle waves shadow the last board, store nothing

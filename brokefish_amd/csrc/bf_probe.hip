@@ -166,3 +166,49 @@ extern "C" double bf_stream_rate(const void* buf, size_t bytes, int workgroups, 
     if (e != hipSuccess || le != hipSuccess) return fail(BF_ERR_LAUNCH, hipGetErrorString(e != hipSuccess ? e : le));
     return (double)bytes * workgroups * reps / ((double)ms * 1e-3) / 1e12;
 }
+
+// ---- quantiser probe ---------------------------------------------------------------------------
+// The kernels' row quantisers applied to a caller's values with a caller's scale, so that the
+// instruction sequences they are built from (the corrected-reciprocal quotient, the byte-select
+// add, v_cvt_pk_u8_f32, the e4m3 conversion) can be held against rint / clamp on the host.
+#include "bf_device.hip.h"
+
+namespace {
+
+template <int MODE>
+__global__ void quant_probe(const float* x, float scale, long n4, unsigned* out) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n4) return;
+    const float4 v = reinterpret_cast<const float4*>(x)[i];
+    const float inv = 1.0f / scale;
+    unsigned w;
+    if constexpr (MODE == BF_PROBE_S8) w = bf::quant4<false>(v.x, v.y, v.z, v.w, scale, inv);
+    else if constexpr (MODE == BF_PROBE_U8_RELU) w = bf::quant4_relu_u8(v.x, v.y, v.z, v.w, scale, inv);
+    else w = bf::quant4<true>(v.x, v.y, v.z, v.w, scale, inv);
+    out[i] = w;
+}
+
+}  // namespace
+
+extern "C" int bf_quant_probe(int mode, const float* x, float scale, int64_t n, uint8_t* out, void* stream) {
+    if (!x || !out || n < 4 || (n & 3) || ((uintptr_t)x & 15) || ((uintptr_t)out & 3) || !(scale > 0.0f)) {
+        bf::set_error("bf_quant_probe: x (16-byte aligned) and out (4-byte aligned) must not be NULL, n a positive multiple of 4, scale > 0");
+        return BF_ERR_ARGUMENT;
+    }
+    const long n4 = n / 4;
+    const dim3 grid((unsigned)((n4 + 255) / 256)), block(256);
+    hipStream_t s = (hipStream_t)stream;
+    unsigned* o = reinterpret_cast<unsigned*>(out);
+    if (mode == BF_PROBE_S8) hipLaunchKernelGGL(quant_probe<BF_PROBE_S8>, grid, block, 0, s, x, scale, n4, o);
+    else if (mode == BF_PROBE_U8_RELU) hipLaunchKernelGGL(quant_probe<BF_PROBE_U8_RELU>, grid, block, 0, s, x, scale, n4, o);
+    else if (mode == BF_PROBE_E4M3) hipLaunchKernelGGL(quant_probe<BF_PROBE_E4M3>, grid, block, 0, s, x, scale, n4, o);
+    else {
+        bf::set_error("bf_quant_probe: mode must be BF_PROBE_S8, BF_PROBE_U8_RELU or BF_PROBE_E4M3");
+        return BF_ERR_ARGUMENT;
+    }
+    if (hipGetLastError() != hipSuccess) {
+        bf::set_error("bf_quant_probe: launch failed");
+        return BF_ERR_LAUNCH;
+    }
+    return BF_OK;
+}

@@ -167,6 +167,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         return std::pair<double, double>{s8, u8};
     }, "the s8 and u8 quantisation maxima compiled into the library");
     m.def("fp8_q_max", []() { return bf_fp8_q_max(); }, "what a row's largest magnitude maps to in e4m3");
+    m.def("abi_tag", []() { return (uint64_t)BF_ABI_TAG; }, "interface tag of the header this module was compiled against");
+    m.def("library_abi_tag", []() { return bf_abi_tag(); }, "interface tag of the library this module is linked to");
     m.def("kernel_choice", [](int64_t d_model, int64_t n_layers, int64_t n_heads, int64_t d_ff, int64_t n_value, int64_t n,
                               int64_t quant, int64_t kernel, bool board_blobs) {
         bf_eval_args a{};

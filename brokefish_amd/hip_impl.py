@@ -120,6 +120,14 @@ def load_library():
         L.bf_mfma_rate.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p]
         L.bf_stream_rate.restype = C.c_double
         L.bf_stream_rate.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        L.bf_quant_probe.restype = C.c_int
+        L.bf_quant_probe.argtypes = [C.c_int, C.c_void_p, C.c_float, C.c_int64, C.c_void_p, C.c_void_p]
+        L.bf_abi_tag.restype = C.c_uint64
+        # the ctypes mirror of bf_eval_args must be the struct the library was compiled with: a
+        # shorter one would make the library read pointers from beyond it
+        if (L.bf_abi_tag() & 0xFFFFFFFF) != C.sizeof(_Args):
+            raise RuntimeError(f"{path} was built with a bf_eval_args of {L.bf_abi_tag() & 0xFFFFFFFF} bytes, this binding "
+                               f"passes {C.sizeof(_Args)}: rebuild the library (`__graft_entry__.build()`)")
         _lib = L
     return _lib
 
@@ -139,6 +147,12 @@ def load_extension():
         except ImportError as e:
             raise RuntimeError(f"the PyTorch extension module is not built ({e}); build it with "
                                "`python -c 'import __graft_entry__ as g; g.build()'`") from e
+        # the module was compiled against one version of the header and is linked to whatever
+        # library file is in the tree now: refuse a pair that does not belong together
+        if _bf_torch.abi_tag() != _bf_torch.library_abi_tag():
+            raise RuntimeError("brokefish_amd/_bf_torch.so was built for another version of libbrokefish_hip.so "
+                               f"(interface tag {_bf_torch.abi_tag():#x} against {_bf_torch.library_abi_tag():#x}): "
+                               "rebuild it (`brokefish_amd._build.build_torch_ext()`) or use binding='ctypes'")
         _ext = _bf_torch
     return _ext
 
@@ -226,6 +240,24 @@ def _check_leaves(leaves, n, device):
             count.numel() != 1 or index.device != device or count.device != device or not index.is_contiguous():
         raise ValueError(f"leaves must be (index [{n}] int32, count [1] int32) on {device}")
     return index, count
+
+
+def quant_probe(x, scale: float, mode: str = "s8"):
+    """The kernels' row quantiser on its own (``bf_quant_probe``): ``x`` float32 on the GPU, its
+    length a multiple of 4 -> the operand bytes for activation scale ``scale``.  ``mode``: "s8"
+    (signed int8), "u8_relu" (the unsigned hidden-row quantiser with the ReLU folded in) or "e4m3"."""
+    modes = {"s8": 0, "u8_relu": 1, "e4m3": 2}
+    if mode not in modes or x.dtype is not torch.float32 or not x.is_cuda or x.dim() != 1 or x.numel() % 4:
+        raise ValueError("x must be a float32 vector on the GPU with a multiple of 4 elements; mode one of " + ", ".join(modes))
+    x = x.contiguous()
+    out = torch.empty(x.numel(), dtype=torch.uint8, device=x.device)
+    lib = load_library()
+    with torch.cuda.device(x.device):
+        rc = lib.bf_quant_probe(modes[mode], x.data_ptr(), float(scale), x.numel(), out.data_ptr(),
+                                C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream))
+    if rc:
+        raise RuntimeError(f"bf_quant_probe failed ({rc}): {lib.bf_last_error().decode()}")
+    return out
 
 
 def compact_leaves(flags, out=None):

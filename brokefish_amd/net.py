@@ -61,10 +61,12 @@ class BrokefishNet(nn.Module):
     def forward(self, boards, control, rep, mask=None):
         """The master network in plain PyTorch, in the parameters' dtype and on their device
         (reference brokefish/nn/model.py:621-645): ``boards [n,32]`` int16 words, ``control [n]``
-        int16, ``rep [n]`` uint8 -> ``(policy [n,32,64], promo [n,32,4], value [n])``; with ``mask``
-        ([n,32] int64 legal-move words) illegal policy entries are -inf.  This is what a trainer
-        differentiates and what :func:`brokefish_amd.sync.check_weights_propagate` holds a packed
-        evaluator against; the evaluator itself never calls it."""
+        int16, ``rep [n]`` uint8 -> ``(policy [n,32,64], promo [n,32,4], value [n])``, raw logits.
+        ``mask`` is accepted and ignored, as in the reference (rule features are not carried here,
+        and without them its ``forward`` never reads the mask: "a caller may always pass what it
+        has"); :meth:`forward_masked` is the variant that sets illegal entries to -inf.  This is
+        what a trainer differentiates and what :func:`brokefish_amd.sync.check_weights_propagate`
+        holds a packed evaluator against; the evaluator itself never calls it."""
         w = boards.to(torch.int64) & 0xFFFF
         alive = ((w >> 11) & 1) == 0
         stm = (control < 0).to(torch.int64)
@@ -96,11 +98,15 @@ class BrokefishNet(nn.Module):
             value = pr[:, 2] - pr[:, 0]
         if self.value_head != "king":           # the pooled heads predict in White's frame
             value = torch.where(control > 0, value, -value)
-        policy = self.policy(h)
-        if mask is not None:
-            legal = ((mask.to(torch.int64)[..., None] >> torch.arange(64, device=mask.device)) & 1).bool()
-            policy = policy.masked_fill(~legal, float("-inf"))
-        return policy, self.promo(h), value
+        return self.policy(h), self.promo(h), value
+
+    def forward_masked(self, boards, control, rep, mask):
+        """``forward`` with the illegal policy entries set to -inf (``mask [n,32]`` int64 legal-move
+        words, bit s of word p set iff p -> s is legal): what the evaluator's ``forward_masked``
+        returns, for comparisons; not for a loss (0 * -inf is NaN)."""
+        policy, promo, value = self.forward(boards, control, rep)
+        legal = ((mask.to(torch.int64)[..., None] >> torch.arange(64, device=mask.device)) & 1).bool()
+        return policy.masked_fill(~legal, float("-inf")), promo, value
 
     @torch.no_grad()
     def randomise_layers_(self, seed: int = 1, scale: float = 1.0) -> "BrokefishNet":

@@ -187,6 +187,16 @@ typedef struct {
     const int32_t* leaf_count;
 } bf_eval_args;
 
+/* Binary interface of this header.  BF_ABI_VERSION is raised whenever a struct or a signature of
+ * this header changes; bf_abi_tag() returns (BF_ABI_VERSION << 32) | sizeof(bf_eval_args) as the
+ * LIBRARY was compiled.  A binding compiled against this header compares that with its own
+ * BF_ABI_TAG before its first call and refuses a library it was not built for (a shorter
+ * bf_eval_args would make the library read pointers from beyond the caller's struct).  No
+ * counterpart in the reference, whose module and kernels are one compilation. */
+#define BF_ABI_VERSION 4
+#define BF_ABI_TAG (((uint64_t)BF_ABI_VERSION << 32) | (uint64_t)sizeof(bf_eval_args))
+uint64_t bf_abi_tag(void);
+
 /* Largest n for which AUTO prefers OCTO over DUO / TWIN on the 256-wide network. */
 int64_t bf_board_max_n(void);
 /* The kernel AUTO would run for these arguments (enum bf_kernel), or a negative bf_status. */
@@ -251,6 +261,18 @@ double bf_mfma_rate(int quant, int* scratch, int iters, int reps, void* stream);
  * equal 32-bit words.  Returns a negative bf_status on error.  Synchronises the stream.
  * No counterpart in the reference. */
 double bf_stream_rate(const void* buf, size_t bytes, int workgroups, int reps, int* sink, void* stream);
+
+/* The kernels' row quantisers on their own, for tests: out[i] = the byte the evaluator would write
+ * for x[i] under the activation scale `scale` (n a multiple of 4, x 16-byte aligned DEVICE memory).
+ *   BF_PROBE_S8       signed int8: rint(x / scale) as a correctly rounded quotient, low byte kept
+ *                     (the row scale keeps |x / scale| <= 127; nothing clamps here)
+ *   BF_PROBE_U8_RELU  the unsigned quantiser of the feed-forward hidden row with the ReLU folded
+ *                     in: rint(max(x, 0) / scale) saturated to [0, 255]
+ *   BF_PROBE_E4M3     OCP e4m3 code of x / scale clamped to +-448
+ * The device twin of the reference's quantiser unit tests (reference csrc/tests/tint8.cu:39-61,
+ * :190-227).  Asynchronous on `stream`. */
+enum bf_probe_mode { BF_PROBE_S8 = 0, BF_PROBE_U8_RELU = 1, BF_PROBE_E4M3 = 2 };
+int bf_quant_probe(int mode, const float* x, float scale, int64_t n, uint8_t* out, void* stream);
 
 /* In-kernel phase accounting, the counterpart of the reference's profile hooks
  * (reference csrc/encoder.cu:1083-1177 and :1886-1903: set_profile / read_profile /

@@ -43,6 +43,8 @@ int main(void) {
     if (bf_compact_leaves(NULL, 4, NULL, NULL, NULL) != BF_ERR_ARGUMENT) return 17;
     if (bf_mfma_rate(BF_QUANT_INT8, NULL, 10, 1, NULL) >= 0.0) return 14;
     if (bf_stream_rate(NULL, 32768, 4, 1, NULL, NULL) >= 0.0) return 18;
+    if (bf_abi_tag() != BF_ABI_TAG || (bf_abi_tag() >> 32) != BF_ABI_VERSION) return 19;    /* this client and the library agree */
+    if (bf_quant_probe(BF_PROBE_S8, NULL, 1.0f, 4, NULL, NULL) != BF_ERR_ARGUMENT) return 20;
     printf("abi ok: %s\n", bf_last_error());
     return 0;
 }

@@ -48,6 +48,22 @@ def test_header_is_plain_c_and_a_c_client_links_and_gets_statuses(tmp_path):
     assert run.stdout.startswith("abi ok")
 
 
+def test_interface_tag_ties_the_bindings_to_the_library():
+    # a binding built for another version of the header must not reach the library: the ctypes
+    # mirror of bf_eval_args is checked on load, the extension module compares its compiled-in tag
+    lib = hip_impl.load_library()
+    tag = lib.bf_abi_tag()
+    header = open(os.path.join(ROOT, "include", "brokefish_hip.h")).read()
+    assert tag >> 32 == int(re.search(r"#define BF_ABI_VERSION (\d+)", header).group(1))
+    assert tag & 0xFFFFFFFF == ctypes.sizeof(hip_impl._Args)
+    if os.path.exists(_build.TORCH_EXT):
+        ext = hip_impl.load_extension()
+        assert ext.abi_tag() == ext.library_abi_tag() == tag
+    # building the library removes an extension module that was built against the previous one
+    src = open(os.path.join(os.path.dirname(_build.__file__), "_build.py")).read()
+    assert "os.remove(TORCH_EXT)" in src[src.index("def build_hip"):src.index("def build_chessgen")]
+
+
 def test_constants_agree_between_host_and_library():
     # the counterpart of the reference's Python<->CUDA constant pin (tests/test_quant.py:233-269)
     assert hip_impl.int8_q_max() == (hip_impl.Q_MAX_S8, hip_impl.Q_MAX_U8) == (127.0, 255.0)

@@ -239,6 +239,49 @@ def test_compacted_leaf_list_with_a_device_side_count_equals_the_flag_route(base
     assert (edges["n_edges"][1::2] == 0).all() and (edges["n_edges"][0::2] > 0).any()
 
 
+@pytest.mark.parametrize("n", [5000, 65536])
+def test_compaction_of_more_flags_than_one_pass_holds(n):
+    # the compaction kernel walks the flags 1024 at a time, carrying the count from pass to pass
+    from brokefish_amd import hip_impl
+    g = torch.Generator().manual_seed(n)
+    for flags in (torch.rand(n, generator=g) < 0.37, torch.ones(n, dtype=torch.bool), torch.arange(n) == n - 1,
+                  torch.arange(n) % 1024 == 1023, torch.zeros(n, dtype=torch.bool)):
+        index, count = hip_impl.compact_leaves(flags.cuda())
+        k = int(flags.sum())
+        assert int(count.item()) == k
+        assert torch.equal(index[:k].cpu().long(), flags.nonzero()[:, 0])
+    # uint8 flags with values other than 1 count as set; a reused output pair keeps its tail
+    f8 = (torch.arange(n) % 5 == 0).to(torch.uint8) * 200
+    out = hip_impl.compact_leaves(torch.ones(n, dtype=torch.bool).cuda())
+    index, count = hip_impl.compact_leaves(f8.cuda(), out=out)
+    k = int((f8 != 0).sum())
+    assert int(count.item()) == k and torch.equal(index[:k].cpu().long(), f8.nonzero()[:, 0])
+    assert torch.equal(index[k:].cpu().long(), torch.arange(k, n))
+
+
+@pytest.mark.parametrize("kernel", ["twin", "octo", "duo", "board", "quad"])
+def test_a_leaf_list_entry_that_is_no_position_of_the_launch_is_skipped(base, kernel):
+    # every kernel treats a malformed entry (negative, or past n) like a slot past the count:
+    # nothing is evaluated for it and no row is written
+    net, sd, boards, quad, co = base
+    model = quad if kernel == "quad" else boards[kernel]
+    b, c, r, m = positions.random_positions(37, plies=120, seed=33)
+    bd, cd, rd, md = _dev(b, c, r, m)
+    full = [t.clone() for t in model.forward_full(bd, cd, rd, md)]
+    best = model.best_out.clone()
+    index = torch.tensor([5, -1, 36, 37, 1 << 20, 0, 11] + [0] * 30, dtype=torch.int32).cuda()
+    count = torch.tensor([7], dtype=torch.int32).cuda()
+    for t in (model.policy_out, model.promo_out, model.value_out):
+        t.fill_(7.0)
+    model.best_out.fill_(-7)
+    p, q, v = model.forward_full(bd, cd, rd, md, leaves=(index, count))
+    hit = torch.zeros(37, dtype=torch.bool)
+    hit[[5, 36, 0, 11]] = True
+    hd = hit.cuda()
+    assert torch.equal(p[hd], full[0][hd]) and torch.equal(v[hd], full[2][hd]) and torch.equal(model.best_out[hd], best[hd])
+    assert (v[~hd] == 7.0).all() and (p[~hd] == 7.0).all() and (model.best_out[~hd] == -7).all()
+
+
 def test_full_batch_at_4096_on_the_throughput_kernel(base):
     net, sd, boards, quad, co = base
     auto = encoder_impl("hip")(net, int8=True, out_dtype=torch.float32)

@@ -126,8 +126,9 @@ def test_master_network_forward_is_the_fp32_restatement_and_the_references_golde
             assert np.abs(got[2].numpy()[:nb] - golden[f"fp32_value_nv{nv}"]).max() < 2e-6
     m = torch.full((8, 32), 0x0F0F, dtype=torch.int64)
     with torch.no_grad():
-        pm = net(b, c, r, mask=m)[0]
-    assert torch.isneginf(pm[:, :, 4]).all() and torch.isfinite(pm[:, :, 0]).all()
+        raw, pm, plain = net(b, c, r, mask=m)[0], net.forward_masked(b, c, r, m)[0], net(b, c, r)[0]
+    assert torch.isfinite(raw).all() and torch.equal(raw, plain)                 # forward ignores the mask, as the reference's
+    assert torch.isneginf(pm[:, :, 4]).all() and torch.equal(pm[:, :, 0], raw[:, :, 0])
 
 
 @pytest.mark.gpu
