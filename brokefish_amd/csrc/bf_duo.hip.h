@@ -38,6 +38,7 @@ using board::lds_barrier;
 using board::tapbits;
 using board::wait_vm;
 
+template <bool FP8>
 struct Cfg : Layout<256> {
     static constexpr int NP = 2, NW = 8;
     static constexpr int XS = NP * NW * 64;               // floats of one exchange slot
@@ -45,7 +46,10 @@ struct Cfg : Layout<256> {
     static constexpr int HID_OFF = XCH_OFF + 3 * XS * 4;
     static constexpr int HID_P = (F / 32) * FRAG;         // a position's hidden row
     static constexpr int ACT_OFF = HID_OFF + NP * HID_P;
-    static constexpr int ACT_P = NT * FRAG;               // a position's row of the width
+    // a position's quantised row of the width: operand bytes; in the e4m3 format widened to fp16 on
+    // the way in (every e4m3 value is an fp16 value), so that the products read ready-made operands
+    static constexpr int ACT_FRAG = FP8 ? 2 * FRAG : FRAG;
+    static constexpr int ACT_P = NT * ACT_FRAG;
     static constexpr int PAR_OFF = ACT_OFF + NP * ACT_P;
     static constexpr int PWL_FLOATS = A_FLOATS + B_FLOATS;
     static constexpr int TOK_OFF = PAR_OFF + 4 * PWL_FLOATS * 4;   // activation scale of every token, per position
@@ -54,9 +58,18 @@ struct Cfg : Layout<256> {
     static_assert(NT * 4 * FRAG <= HID_P, "normalised stream overlay");
 };
 
+// one 16-deep step on operands already widened to fp16; int8 builds never call it
+template <bool SWAP>
+__device__ __forceinline__ v16f f16_step(const v8h& w, const v8h& act, const v16f& acc) {
+    return SWAP ? __builtin_amdgcn_mfma_f32_32x32x16_f16(act, w, acc, 0, 0, 0)
+                : __builtin_amdgcn_mfma_f32_32x32x16_f16(w, act, acc, 0, 0, 0);
+}
+template <bool SWAP>
+__device__ __forceinline__ v16i f16_step(const v8h&, const v8h&, const v16i& acc) { return acc; }
+
 template <bool TAPS, bool FP8, bool PROF = false>
 __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
-    typedef Cfg C;
+    typedef Cfg<FP8> C;
     typedef typename Acc<FP8>::type acc_t;
     constexpr int NP = C::NP, D = C::D, F = C::F, NT = C::NT, TW = C::TW, CW = C::CW, KCF = C::KCF;
     constexpr int STEPS = C::STEPS, BPW = C::BPW, HB = C::HB;
@@ -247,7 +260,14 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
 #pragma unroll
             for (int j = 0; j < 4; j++)
                 w[j] = (int)quant4<FP8>(y[p][4 * j], y[p][4 * j + 1], y[p][4 * j + 2], y[p][4 * j + 3], sa[p], inv);
-            *reinterpret_cast<v4i*>(act + p * C::ACT_P + tile * FRAG + lane * 16) = w;
+            if constexpr (FP8) {
+                const v2l wl = __builtin_bit_cast(v2l, w);
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    *reinterpret_cast<v8h*>(act + p * C::ACT_P + (2 * tile + h) * FRAG + lane * 16) = e4m3x8_as_f16(wl[h]);
+            } else {
+                *reinterpret_cast<v4i*>(act + p * C::ACT_P + tile * FRAG + lane * 16) = w;
+            }
             if (TAPS && tap && live[p])
 #pragma unroll
                 for (int j = 0; j < 4; j++)
@@ -357,6 +377,41 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             if ((p) == 1 && s_ == 3) fetch_half(2 * (k) + NSETS, lbase, lfollow);                    \
         }                                                                                            \
     } while (0)
+        // e4m3: both positions' products with the wave's k-th block, step by step.  A weight fragment is
+        // widened to fp16 once and multiplied with both positions' operands; these come from LDS
+        // already widened (A16: the row of the width) or as bytes (the hidden row).  Each accumulator
+        // sees its sixteen 16-deep steps in order, as in the other kernels.
+#define BF_DUO_PAIR_F8(SWAP, k, A16, B0, B1, R)                                                      \
+    do {                                                                                             \
+        const uint8_t* const bp_[2] = {(B0), (B1)};                                                  \
+        fetch_half(2 * (k) + NSETS - 1, lbase, lfollow);                                             \
+        (R)[0] = zero;                                                                               \
+        (R)[1] = zero;                                                                               \
+        /* the operands of a step are fetched from LDS one step ahead: [position][half] */           \
+        v4i cur_[2][2], nxt_[2][2];                                                                  \
+        _Pragma("unroll") for (int p_ = 0; p_ < 2; p_++)                                             \
+            _Pragma("unroll") for (int h_ = 0; h_ < ((A16) ? 2 : 1); h_++)                           \
+                cur_[p_][h_] = ldsfrag(bp_[p_] + ((A16) ? h_ : 0) * FRAG);                           \
+        _Pragma("unroll") for (int s_ = 0; s_ < 8; s_++) {                                           \
+            _Pragma("unroll") for (int p_ = 0; p_ < 2; p_++)                                         \
+                _Pragma("unroll") for (int h_ = 0; h_ < ((A16) ? 2 : 1); h_++)                       \
+                    nxt_[p_][h_] = s_ + 1 < 8 ? ldsfrag(bp_[p_] + ((A16) ? 2 * (s_ + 1) + h_ : s_ + 1) * FRAG) : cur_[p_][h_]; \
+            const v2l wl_ = __builtin_bit_cast(v2l, frt[(2 * (k) + s_ / 4) % NSETS][s_ % 4]);        \
+            _Pragma("unroll") for (int h_ = 0; h_ < 2; h_++) {                                       \
+                const v8h wh_ = e4m3x8_as_f16(wl_[h_]);                                              \
+                _Pragma("unroll") for (int p_ = 0; p_ < 2; p_++) {                                   \
+                    v8h ah_;                                                                         \
+                    if (A16) ah_ = __builtin_bit_cast(v8h, cur_[p_][h_]);                            \
+                    else ah_ = e4m3x8_as_f16(__builtin_bit_cast(v2l, cur_[p_][0])[h_]);              \
+                    (R)[p_] = f16_step<SWAP>(wh_, ah_, (R)[p_]);                                     \
+                }                                                                                    \
+            }                                                                                        \
+            __builtin_amdgcn_sched_barrier(0);                                                       \
+            _Pragma("unroll") for (int p_ = 0; p_ < 2; p_++)                                         \
+                _Pragma("unroll") for (int h_ = 0; h_ < ((A16) ? 2 : 1); h_++) cur_[p_][h_] = nxt_[p_][h_]; \
+            if (s_ == 3) fetch_half(2 * (k) + NSETS, lbase, lfollow);                                \
+        }                                                                                            \
+    } while (0)
         const acc_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         auto none = [&](int) {};
         const uint8_t* const act1 = act0 + C::ACT_P;
@@ -415,17 +470,34 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             auto ek1 = [&](int s) { epi_k(1, s); };
             auto ev0 = [&](int s) { epi_v(0, s); };
             load_tile16(pA + C::A_BQ + 32 * sub, g, bq);
-            BF_DUO_CHAIN(false, 0, 0, act0, zero, acc[0], none);
-            BF_DUO_CHAIN(false, 0, 1, act1, zero, acc[1], eq0);
-            load_tile16(pA + C::A_BK + 32 * sub, g, bk);
-            BF_DUO_CHAIN(false, 1, 0, act0, zero, acc[0], eq1);
-            BF_DUO_CHAIN(false, 1, 1, act1, zero, acc[1], ek0);
-            load_tile16(tok, g, stok[0]);
-            BF_DUO_CHAIN(true, 2, 0, act0, zero, acc[0], ek1);
-            load_tile16(tok + 32, g, stok[1]);
-            BF_DUO_CHAIN(true, 2, 1, act1, zero, acc[1], ev0);
+            if constexpr (FP8) {
+                // e4m3: a block's two products share the widening of its weight fragments, the
+                // epilogues of both positions follow
+                BF_DUO_PAIR_F8(false, 0, true, act0, act1, acc);
 #pragma unroll
-            for (int s = 0; s < 8; s++) epi_v(1, s);
+                for (int s = 0; s < 8; s++) { epi_q(0, s); epi_q(1, s); }
+                load_tile16(pA + C::A_BK + 32 * sub, g, bk);
+                BF_DUO_PAIR_F8(false, 1, true, act0, act1, acc);
+#pragma unroll
+                for (int s = 0; s < 8; s++) { epi_k(0, s); epi_k(1, s); }
+                load_tile16(tok, g, stok[0]);
+                load_tile16(tok + 32, g, stok[1]);
+                BF_DUO_PAIR_F8(true, 2, true, act0, act1, acc);
+#pragma unroll
+                for (int s = 0; s < 8; s++) { epi_v(0, s); epi_v(1, s); }
+            } else {
+                BF_DUO_CHAIN(false, 0, 0, act0, zero, acc[0], none);
+                BF_DUO_CHAIN(false, 0, 1, act1, zero, acc[1], eq0);
+                load_tile16(pA + C::A_BK + 32 * sub, g, bk);
+                BF_DUO_CHAIN(false, 1, 0, act0, zero, acc[0], eq1);
+                BF_DUO_CHAIN(false, 1, 1, act1, zero, acc[1], ek0);
+                load_tile16(tok, g, stok[0]);
+                BF_DUO_CHAIN(true, 2, 0, act0, zero, acc[0], ek1);
+                load_tile16(tok + 32, g, stok[1]);
+                BF_DUO_CHAIN(true, 2, 1, act1, zero, acc[1], ev0);
+#pragma unroll
+                for (int s = 0; s < 8; s++) epi_v(1, s);
+            }
             BF_PHASE(PH_QKV);
 #pragma unroll
             for (int p = 0; p < NP; p++) {
@@ -477,8 +549,14 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                 }
             };
             auto eo0 = [&](int s) { epi_o(0, s); };
-            BF_DUO_CHAIN(false, 3, 0, act0, zero, acc[0], none);
-            BF_DUO_CHAIN(false, 3, 1, act1, zero, acc[1], eo0);
+            if constexpr (FP8) {
+                BF_DUO_PAIR_F8(false, 3, true, act0, act1, acc);
+#pragma unroll
+                for (int s = 0; s < 8; s++) epi_o(0, s);
+            } else {
+                BF_DUO_CHAIN(false, 3, 0, act0, zero, acc[0], none);
+                BF_DUO_CHAIN(false, 3, 1, act1, zero, acc[1], eo0);
+            }
 #pragma unroll
             for (int s = 0; s < 8; s++) epi_o(1, s);
         }
@@ -521,21 +599,27 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                 }
             };
 #pragma unroll
-            for (int i = 0; i < HT; i++)
+            for (int i = 0; i < HT; i++) {
+                load_tile16(pB + C::B_BFF1 + 128 * st + 32 * (HT * sub + i), g, b1[i]);
+                sw1[i] = pB[C::B_SW + 4 * st + HT * sub + i];
+                if constexpr (FP8) {
+                    BF_DUO_PAIR_F8(false, 4 + HT * st + i, true, act0, act1, acc);
 #pragma unroll
-                for (int p = 0; p < NP; p++) {
-                    const int n = NP * i + p;   // product number within the step; the previous one's epilogue runs under it
-                    if (p == 0) {
-                        load_tile16(pB + C::B_BFF1 + 128 * st + 32 * (HT * sub + i), g, b1[i]);
-                        sw1[i] = pB[C::B_SW + 4 * st + HT * sub + i];
+                    for (int s = 0; s < 8; s++) { epi_f(i, 0, s); epi_f(i, 1, s); }
+                } else {
+#pragma unroll
+                    for (int p = 0; p < NP; p++) {
+                        const int n = NP * i + p;   // product number within the step; the previous one's epilogue runs under it
+                        auto between = [&](int s) {
+                            if (n > 0) epi_f((n - 1) / NP, (n - 1) % NP, s);
+                        };
+                        BF_DUO_CHAIN(false, 4 + HT * st + i, p, act0 + p * C::ACT_P, zero, acc[p], between);
                     }
-                    auto between = [&](int s) {
-                        if (n > 0) epi_f((n - 1) / NP, (n - 1) % NP, s);
-                    };
-                    BF_DUO_CHAIN(false, 4 + HT * st + i, p, act0 + p * C::ACT_P, zero, acc[p], between);
                 }
+            }
+            if constexpr (!FP8)
 #pragma unroll
-            for (int s = 0; s < 8; s++) epi_f(HT - 1, NP - 1, s);
+                for (int s = 0; s < 8; s++) epi_f(HT - 1, NP - 1, s);
             // the maxima of consecutive steps go through different exchange slots
             const int xs = (st & 1) ? 0 : 2 * XS;
 #pragma unroll
@@ -601,11 +685,15 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                 }
             };
 #pragma unroll
-            for (int cc = 0; cc < KCF; cc++)
+            for (int cc = 0; cc < KCF; cc++) {
+                if constexpr (FP8) {
+                    BF_DUO_PAIR_F8(false, 4 + HT * STEPS + cc, false, hid0 + 8 * cc * FRAG, hid0 + C::HID_P + 8 * cc * FRAG, acc);
 #pragma unroll
-                for (int p = 0; p < NP; p++) {
-                    const int n = NP * cc + p;
-                    if constexpr (!FP8)
+                    for (int s = 0; s < 8; s++) { epi_2(cc, 0, s); epi_2(cc, 1, s); }
+                } else {
+#pragma unroll
+                    for (int p = 0; p < NP; p++) {
+                        const int n = NP * cc + p;
                         if (p == 0) {
                             v4i w0[4];
                             load_tile16i(pB + C::B_WSUM + cc * CW + 32 * sub, g, w0);
@@ -614,13 +702,16 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
 #pragma unroll
                                 for (int k = 0; k < 4; k++) init[4 * j + k] = w0[j][k];
                         }
-                    auto between = [&](int s) {
-                        if (n > 0) epi_2((n - 1) / NP, (n - 1) % NP, s);
-                    };
-                    BF_DUO_CHAIN(false, 4 + HT * STEPS + cc, p, hid0 + p * C::HID_P + 8 * cc * FRAG, init, acc[p], between);
+                        auto between = [&](int s) {
+                            if (n > 0) epi_2((n - 1) / NP, (n - 1) % NP, s);
+                        };
+                        BF_DUO_CHAIN(false, 4 + HT * STEPS + cc, p, hid0 + p * C::HID_P + 8 * cc * FRAG, init, acc[p], between);
+                    }
                 }
+            }
+            if constexpr (!FP8)
 #pragma unroll
-            for (int s = 0; s < 8; s++) epi_2(KCF - 1, NP - 1, s);
+                for (int s = 0; s < 8; s++) epi_2(KCF - 1, NP - 1, s);
             v4f b2[4];
             load_tile16(pB + C::B_BFF2 + 32 * sub, g, b2);
             const float sw = pB[C::B_SW + 16 + sub];
@@ -640,6 +731,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         }
         BF_PHASE(PH_FF2);
 #undef BF_DUO_CHAIN
+#undef BF_DUO_PAIR_F8
         if (TAPS && a.taps.resid)
 #pragma unroll
             for (int p = 0; p < NP; p++)
@@ -839,7 +931,7 @@ template <bool TAPS, bool FP8 = false, bool PROF = false>
 hipError_t launch_duo(const KArgs& k, hipStream_t stream) {
     // more than 64 KiB of dynamic LDS has to be requested once per kernel and device
     static std::atomic<unsigned long long> lds_set{0};
-    constexpr int lds_bytes = Cfg::LDS_BYTES;
+    constexpr int lds_bytes = Cfg<FP8>::LDS_BYTES;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return hipErrorInvalidDevice;
     const unsigned long long bit = dev < 64 ? 1ull << dev : 0;

@@ -421,6 +421,42 @@ def test_pooled_value_heads_bit_exact_on_every_kernel(head, nv):
         assert _bits_equal(vw, ww["value"]), kernel
 
 
+@pytest.mark.parametrize("head", ["pooled", "prenorm"])
+@pytest.mark.parametrize("nv", [1, 3])
+def test_pooled_value_heads_in_the_e4m3_format(head, nv):
+    # the value heads are fp32 arithmetic behind either operand format: in e4m3 the kernels must
+    # agree with each other bit for bit, give the emulation's value when started from the emulation's
+    # own final residual stream, and follow it free-running wherever no byte flipped at a tie
+    from oracle import emulated
+    torch.manual_seed(2)
+    net = BrokefishNet(n_value=nv, value_head=head).eval().randomise_layers_(seed=7)
+    sd = {k: v.detach() for k, v in net.state_dict().items()}
+    b, c, r, m = positions.random_positions(64, plies=120, seed=19, stamp_queen=True)
+    assert (c < 0).any() and (c > 0).any()
+    bd, cd, rd, md = _dev(b, c, r, m)
+    etaps = {}
+    with torch.no_grad():
+        emu = emulated.forward(sd, b, c, r, mode="e4m3", taps=etaps)
+    outs = {}
+    for kernel in ("twin", "octo", "duo", "board"):
+        model = encoder_impl("hip")(net, fp8=True, out_dtype=torch.float32, kernel=kernel)
+        assert model.vmode == {"pooled": 1, "prenorm": 2}[head]
+        outs[kernel] = [t.clone() for t in model.forward_masked(bd, cd, rd, md)]
+        for x, y in zip(outs[kernel], outs["twin"]):
+            assert torch.equal(x, y), kernel
+    forced = model.forward_taps(bd, cd, rd, x_in=etaps["resid"][7].cuda(), layer_begin=8, layer_end=8, want=["normed"])
+    assert (forced["value"].cpu() - emu[2]).abs().max() < 1e-5
+    assert (forced["policy"].cpu() - emu[0]).abs().max() < 1e-4
+    dv = (outs["twin"][2].cpu() - emu[2]).abs()
+    assert (dv < 2e-2).float().mean() > 0.5 and dv.max() < 0.5 and (outs["twin"][2].abs() <= 1).all()
+    # Black to move flips the sign of the White-frame prediction: the same board under the other
+    # mover gives a value of the other sign from these heads only through the control word
+    king = BrokefishNet(n_value=nv).eval()
+    king.load_state_dict({k: v for k, v in sd.items() if k != "value_mode"})
+    vk = encoder_impl("hip")(king, fp8=True, out_dtype=torch.float32).forward_full(bd, cd, rd)[2]
+    assert not torch.allclose(vk, outs["twin"][2], atol=1e-3)
+
+
 def test_matrix_pipe_probe_reports_a_plausible_rate():
     # a register-resident MFMA loop cannot beat the datasheet peak (5.0 POP/s dense int8 / fp8)
     # and, on a healthy part, reaches most of it; the evaluator's own rate must lie below it
