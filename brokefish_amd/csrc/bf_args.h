@@ -147,8 +147,6 @@ hipError_t launch_twin256_fp8_taps(const KArgs& k, hipStream_t stream);
 // one position per workgroup of eight wavefronts (two per quarter of the width), one workgroup
 // per compute unit: the lowest latency per position for the 256-wide network (int8, e4m3), and
 // the faster form for the 512-wide one (int8)
-hipError_t launch_octo256(const KArgs& k, hipStream_t stream);
-hipError_t launch_octo256_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo256_fp8(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo256_fp8_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512(const KArgs& k, hipStream_t stream);
@@ -161,8 +159,12 @@ hipError_t launch_duo256_fp8(const KArgs& k, hipStream_t stream);
 hipError_t launch_duo256_fp8_taps(const KArgs& k, hipStream_t stream);
 // the int8 builds that carry the phase profile
 hipError_t launch_twin256_prof(const KArgs& k, hipStream_t stream);
-hipError_t launch_octo256_prof(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512_prof(const KArgs& k, hipStream_t stream);
 hipError_t launch_duo256_prof(const KArgs& k, hipStream_t stream);
+// the same kernel with one position per workgroup (the eight-wavefront form for launches that
+// cannot fill the GPU): int8, 256-wide network
+hipError_t launch_solo256(const KArgs& k, hipStream_t stream);
+hipError_t launch_solo256_taps(const KArgs& k, hipStream_t stream);
+hipError_t launch_solo256_prof(const KArgs& k, hipStream_t stream);
 
 }  // namespace bf

@@ -38,9 +38,9 @@ using board::lds_barrier;
 using board::tapbits;
 using board::wait_vm;
 
-template <bool FP8>
+template <bool FP8, int NP_>
 struct Cfg : Layout<256> {
-    static constexpr int NP = 2, NW = 8;
+    static constexpr int NP = NP_, NW = 8;   // positions per workgroup (2; 1: the latency form), wavefronts
     static constexpr int XS = NP * NW * 64;               // floats of one exchange slot
     static constexpr int XCH_OFF = 0;
     static constexpr int HID_OFF = XCH_OFF + 3 * XS * 4;
@@ -67,9 +67,10 @@ __device__ __forceinline__ v16f f16_step(const v8h& w, const v8h& act, const v16
 template <bool SWAP>
 __device__ __forceinline__ v16i f16_step(const v8h&, const v8h&, const v16i& acc) { return acc; }
 
-template <bool TAPS, bool FP8, bool PROF = false>
+template <bool TAPS, bool FP8, bool PROF = false, int NPOS = 2>
 __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
-    typedef Cfg<FP8> C;
+    typedef Cfg<FP8, NPOS> C;
+    static_assert(NPOS == 2 || (NPOS == 1 && !FP8), "one position per workgroup: the int8 format");
     typedef typename Acc<FP8>::type acc_t;
     constexpr int NP = C::NP, D = C::D, F = C::F, NT = C::NT, TW = C::TW, CW = C::CW, KCF = C::KCF;
     constexpr int STEPS = C::STEPS, BPW = C::BPW, HB = C::HB;
@@ -89,17 +90,19 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
     const int tile = TW * q + sub;   // the tile of the width (and the head) this wave owns
     const int t = lane & 31, g = lane >> 5;
 
-    // the two positions of this workgroup: its own pair, or entries 2 blockIdx.x and 2 blockIdx.x + 1
-    // of the compacted leaf list.  A slot without a position (past the end, skipped, not in this
-    // launch) computes its neighbour's position again and stores nothing; a workgroup without any
-    // position leaves before the first barrier.
+    // the positions of this workgroup: its own NP slots of the launch, or those entries of the
+    // compacted leaf list.  A slot without a position (past the end, skipped, not in this launch)
+    // computes its neighbour's position again and stores nothing; a workgroup without any position
+    // leaves before the first barrier.
     int bp[NP];
     bool live[NP];
     {
         const int cnt = a.leaf_index ? *a.leaf_count : a.n;
+        bool any = false;
+        int some = 0;
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            const int j = 2 * (int)blockIdx.x + p;
+            const int j = NP * (int)blockIdx.x + p;
             int b = j;
             bool ok = j < cnt;
             if (a.leaf_index) {
@@ -109,10 +112,12 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             if (ok && a.active) ok = a.active[b] != 0;
             bp[p] = ok ? b : 0;
             live[p] = ok;
+            if (ok) { any = true; some = b; }
         }
-        if (!live[0] && !live[1]) return;
-        if (!live[1]) bp[1] = bp[0];
-        if (!live[0]) bp[0] = bp[1];
+        if (!any) return;
+#pragma unroll
+        for (int p = 0; p < NP; p++)
+            if (!live[p]) bp[p] = some;
     }
     const int nl_run = a.l1 - a.l0;
     // Phase accounting (PROF builds only): the shader clock is read at phase boundaries and the
@@ -374,7 +379,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             (R) = frag_mma<SWAP>(frt[(2 * (k) + s_ / 4) % NSETS][s_ % 4], ring_[s_ % (A_ + 1)], (R)); \
             BETWEEN(s_);                                                                             \
             __builtin_amdgcn_sched_barrier(0);                                                       \
-            if ((p) == 1 && s_ == 3) fetch_half(2 * (k) + NSETS, lbase, lfollow);                    \
+            if ((p) == NP - 1 && s_ == 3) fetch_half(2 * (k) + NSETS, lbase, lfollow);               \
         }                                                                                            \
     } while (0)
         // e4m3: both positions' products with the wave's k-th block, step by step.  A weight fragment is
@@ -436,67 +441,70 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             float qf[NP][16], kf[NP][16], vf[NP][16];
             const float swq = pA[C::A_SW + sub], swk = pA[C::A_SW + TW + sub], swv = pA[C::A_SW + 2 * TW + sub];
             const float bv = pA[C::A_BV + 32 * sub + t];
-            acc_t acc[NP];
+            acc_t acc[2];   // product n of a sequence uses accumulator n & 1; the previous one's epilogue runs under it
             v4f bq[4], bk[4], stok[NP][4];
             // the epilogues, two accumulator registers at a time (slice s of eight)
-            auto epi_q = [&](int p, int s) {
+            auto epi_q = [&](int p, int s, int ai) {
 #pragma unroll
                 for (int e = 2 * s; e < 2 * s + 2; e++) {
-                    qf[p][e] = accf(acc[p], e) * sa[p] * swq + bq[e / 4][e % 4];
+                    qf[p][e] = accf(acc[ai], e) * sa[p] * swq + bq[e / 4][e % 4];
                     if (TAPS && a.taps.acc_qkv && live[p])
-                        a.taps.acc_qkv[(bl[p] * T + t) * 3 * D + 32 * tile + ch(e, g)] = tapbits<false>(acc[p], e);
+                        a.taps.acc_qkv[(bl[p] * T + t) * 3 * D + 32 * tile + ch(e, g)] = tapbits<false>(acc[ai], e);
                 }
             };
-            auto epi_k = [&](int p, int s) {
+            auto epi_k = [&](int p, int s, int ai) {
 #pragma unroll
                 for (int e = 2 * s; e < 2 * s + 2; e++) {
-                    kf[p][e] = accf(acc[p], e) * sa[p] * swk + bk[e / 4][e % 4];
+                    kf[p][e] = accf(acc[ai], e) * sa[p] * swk + bk[e / 4][e % 4];
                     if (TAPS && a.taps.acc_qkv && live[p])
-                        a.taps.acc_qkv[(bl[p] * T + t) * 3 * D + D + 32 * tile + ch(e, g)] = tapbits<false>(acc[p], e);
+                        a.taps.acc_qkv[(bl[p] * T + t) * 3 * D + D + 32 * tile + ch(e, g)] = tapbits<false>(acc[ai], e);
                 }
             };
             // V tile: rows are tokens, so the activation scale is that of token ch(e, g)
-            auto epi_v = [&](int p, int s) {
+            auto epi_v = [&](int p, int s, int ai) {
 #pragma unroll
                 for (int e = 2 * s; e < 2 * s + 2; e++) {
-                    vf[p][e] = accf(acc[p], e) * stok[p][e / 4][e % 4] * swv + bv;
+                    vf[p][e] = accf(acc[ai], e) * stok[p][e / 4][e % 4] * swv + bv;
                     if (TAPS && a.taps.acc_qkv && live[p])
-                        a.taps.acc_qkv[(bl[p] * T + ch(e, g)) * 3 * D + 2 * D + 32 * tile + t] = tapbits<false>(acc[p], e);
+                        a.taps.acc_qkv[(bl[p] * T + ch(e, g)) * 3 * D + 2 * D + 32 * tile + t] = tapbits<false>(acc[ai], e);
                 }
             };
-            auto eq0 = [&](int s) { epi_q(0, s); };
-            auto eq1 = [&](int s) { epi_q(1, s); };
-            auto ek0 = [&](int s) { epi_k(0, s); };
-            auto ek1 = [&](int s) { epi_k(1, s); };
-            auto ev0 = [&](int s) { epi_v(0, s); };
+            auto epi_qkv = [&](int tq, int p, int s, int ai) {
+                if (tq == 0) epi_q(p, s, ai);
+                else if (tq == 1) epi_k(p, s, ai);
+                else epi_v(p, s, ai);
+            };
             load_tile16(pA + C::A_BQ + 32 * sub, g, bq);
             if constexpr (FP8) {
                 // e4m3: a block's two products share the widening of its weight fragments, the
                 // epilogues of both positions follow
                 BF_DUO_PAIR_F8(false, 0, true, act0, act1, acc);
 #pragma unroll
-                for (int s = 0; s < 8; s++) { epi_q(0, s); epi_q(1, s); }
+                for (int s = 0; s < 8; s++) { epi_q(0, s, 0); epi_q(1, s, 1); }
                 load_tile16(pA + C::A_BK + 32 * sub, g, bk);
                 BF_DUO_PAIR_F8(false, 1, true, act0, act1, acc);
 #pragma unroll
-                for (int s = 0; s < 8; s++) { epi_k(0, s); epi_k(1, s); }
+                for (int s = 0; s < 8; s++) { epi_k(0, s, 0); epi_k(1, s, 1); }
                 load_tile16(tok, g, stok[0]);
                 load_tile16(tok + 32, g, stok[1]);
                 BF_DUO_PAIR_F8(true, 2, true, act0, act1, acc);
 #pragma unroll
-                for (int s = 0; s < 8; s++) { epi_v(0, s); epi_v(1, s); }
+                for (int s = 0; s < 8; s++) { epi_v(0, s, 0); epi_v(1, s, 1); }
             } else {
-                BF_DUO_CHAIN(false, 0, 0, act0, zero, acc[0], none);
-                BF_DUO_CHAIN(false, 0, 1, act1, zero, acc[1], eq0);
-                load_tile16(pA + C::A_BK + 32 * sub, g, bk);
-                BF_DUO_CHAIN(false, 1, 0, act0, zero, acc[0], eq1);
-                BF_DUO_CHAIN(false, 1, 1, act1, zero, acc[1], ek0);
-                load_tile16(tok, g, stok[0]);
-                BF_DUO_CHAIN(true, 2, 0, act0, zero, acc[0], ek1);
-                load_tile16(tok + 32, g, stok[1]);
-                BF_DUO_CHAIN(true, 2, 1, act1, zero, acc[1], ev0);
+                // Q, K, V blocks in turn, each for every position: 3 NP products
 #pragma unroll
-                for (int s = 0; s < 8; s++) epi_v(1, s);
+                for (int n = 0; n < 3 * NP; n++) {
+                    const int tq = n / NP, p = n % NP;
+                    if (n == NP) load_tile16(pA + C::A_BK + 32 * sub, g, bk);
+                    if (tq == 2) load_tile16(tok + 32 * p, g, stok[p]);
+                    auto between = [&](int s) {
+                        if (n > 0) epi_qkv((n - 1) / NP, (n - 1) % NP, s, (n - 1) & 1);
+                    };
+                    if (tq == 2) BF_DUO_CHAIN(true, 2, p, act0 + p * C::ACT_P, zero, acc[n & 1], between);
+                    else BF_DUO_CHAIN(false, tq, p, act0 + p * C::ACT_P, zero, acc[n & 1], between);
+                }
+#pragma unroll
+                for (int s = 0; s < 8; s++) epi_v(NP - 1, s, (3 * NP - 1) & 1);
             }
             BF_PHASE(PH_QKV);
 #pragma unroll
@@ -536,29 +544,33 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         {
             float so[NP];
             quant_exchange2(o, so, TAPS ? a.taps.qa_out : nullptr, bl, false);
-            acc_t acc[NP];
+            acc_t acc[2];
             v4f bo[4];
             load_tile16(pA + C::A_BOUT + 32 * sub, g, bo);
             const float sw = pA[C::A_SW + 3 * TW + sub];
-            auto epi_o = [&](int p, int s) {
+            auto epi_o = [&](int p, int s, int ai) {
 #pragma unroll
                 for (int e = 2 * s; e < 2 * s + 2; e++) {
-                    x[p][e] = x[p][e] + (accf(acc[p], e) * so[p] * sw + bo[e / 4][e % 4]);
+                    x[p][e] = x[p][e] + (accf(acc[ai], e) * so[p] * sw + bo[e / 4][e % 4]);
                     if (TAPS && a.taps.acc_out && live[p])
-                        a.taps.acc_out[(bl[p] * T + t) * D + 32 * tile + ch(e, g)] = tapbits<false>(acc[p], e);
+                        a.taps.acc_out[(bl[p] * T + t) * D + 32 * tile + ch(e, g)] = tapbits<false>(acc[ai], e);
                 }
             };
-            auto eo0 = [&](int s) { epi_o(0, s); };
             if constexpr (FP8) {
                 BF_DUO_PAIR_F8(false, 3, true, act0, act1, acc);
 #pragma unroll
-                for (int s = 0; s < 8; s++) epi_o(0, s);
+                for (int s = 0; s < 8; s++) epi_o(0, s, 0);
             } else {
-                BF_DUO_CHAIN(false, 3, 0, act0, zero, acc[0], none);
-                BF_DUO_CHAIN(false, 3, 1, act1, zero, acc[1], eo0);
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    auto between = [&](int s) {
+                        if (p > 0) epi_o(p - 1, s, (p - 1) & 1);
+                    };
+                    BF_DUO_CHAIN(false, 3, p, act0 + p * C::ACT_P, zero, acc[p & 1], between);
+                }
             }
 #pragma unroll
-            for (int s = 0; s < 8; s++) epi_o(1, s);
+            for (int s = 0; s < 8; s++) epi_o(NP - 1, s, (NP - 1) & 1);
         }
         BF_PHASE(PH_OUT);
 
@@ -581,21 +593,23 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
 #pragma unroll
         for (int st = 0; st < STEPS; st++) {
             float hf[NP][HT][16];
-            float am[NP] = {0.0f, 0.0f};
-            acc_t acc[NP];
+            float am[NP];
+#pragma unroll
+            for (int p = 0; p < NP; p++) am[p] = 0.0f;
+            acc_t acc[2];
             v4f b1[HT][4];
             float sw1[HT];
-            auto epi_f = [&](int i, int p, int s) {
+            auto epi_f = [&](int i, int p, int s, int ai) {
 #pragma unroll
                 for (int e = 2 * s; e < 2 * s + 2; e++) {
                     // int8: the ReLU is the saturation of the unsigned quantiser below, and the
                     // running maximum starts at 0, so negative values need no clamp here
-                    float v = accf(acc[p], e) * sa[p] * sw1[i] + b1[i][e / 4][e % 4];
+                    float v = accf(acc[ai], e) * sa[p] * sw1[i] + b1[i][e / 4][e % 4];
                     if constexpr (FP8) v = __builtin_fmaxf(v, 0.0f);
                     hf[p][i][e] = v;
                     am[p] = __builtin_fmaxf(am[p], v);
                     if (TAPS && a.taps.acc_ff1 && live[p])
-                        a.taps.acc_ff1[(bl[p] * T + t) * F + 512 * st + 128 * q + 32 * (HT * sub + i) + ch(e, g)] = tapbits<false>(acc[p], e);
+                        a.taps.acc_ff1[(bl[p] * T + t) * F + 512 * st + 128 * q + 32 * (HT * sub + i) + ch(e, g)] = tapbits<false>(acc[ai], e);
                 }
             };
 #pragma unroll
@@ -605,21 +619,21 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                 if constexpr (FP8) {
                     BF_DUO_PAIR_F8(false, 4 + HT * st + i, true, act0, act1, acc);
 #pragma unroll
-                    for (int s = 0; s < 8; s++) { epi_f(i, 0, s); epi_f(i, 1, s); }
+                    for (int s = 0; s < 8; s++) { epi_f(i, 0, s, 0); epi_f(i, 1, s, 1); }
                 } else {
 #pragma unroll
                     for (int p = 0; p < NP; p++) {
                         const int n = NP * i + p;   // product number within the step; the previous one's epilogue runs under it
                         auto between = [&](int s) {
-                            if (n > 0) epi_f((n - 1) / NP, (n - 1) % NP, s);
+                            if (n > 0) epi_f((n - 1) / NP, (n - 1) % NP, s, (n - 1) & 1);
                         };
-                        BF_DUO_CHAIN(false, 4 + HT * st + i, p, act0 + p * C::ACT_P, zero, acc[p], between);
+                        BF_DUO_CHAIN(false, 4 + HT * st + i, p, act0 + p * C::ACT_P, zero, acc[n & 1], between);
                     }
                 }
             }
             if constexpr (!FP8)
 #pragma unroll
-                for (int s = 0; s < 8; s++) epi_f(HT - 1, NP - 1, s);
+                for (int s = 0; s < 8; s++) epi_f(HT - 1, NP - 1, s, (NP * HT - 1) & 1);
             // the maxima of consecutive steps go through different exchange slots
             const int xs = (st & 1) ? 0 : 2 * XS;
 #pragma unroll
@@ -663,25 +677,25 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         {
             double o64[NP][16];
             float o32[NP][16];
-            acc_t acc[NP];
+            acc_t acc[2];
             acc_t init = zero;
             float sw2[KCF];   // e4m3: one weight scale per k-chunk
             if constexpr (FP8)
 #pragma unroll
                 for (int cc = 0; cc < KCF; cc++) sw2[cc] = pB[C::B_SW + 16 + sub * KCF + cc];
-            auto epi_2 = [&](int cc, int p, int s) {
+            auto epi_2 = [&](int cc, int p, int s, int ai) {
 #pragma unroll
                 for (int e = 2 * s; e < 2 * s + 2; e++) {
                     if constexpr (FP8) {
-                        const float part = (accf(acc[p], e) * sh[p][cc]) * sw2[cc];
+                        const float part = (accf(acc[ai], e) * sh[p][cc]) * sw2[cc];
                         o32[p][e] = cc == 0 ? part : o32[p][e] + part;
                     } else {
                         const double sc = (double)sh[p][cc];
-                        const int full = accbits(acc[p], e);
+                        const int full = accbits(acc[ai], e);
                         o64[p][e] = cc == 0 ? (double)full * sc : __builtin_fma((double)full, sc, o64[p][e]);
                     }
                     if (TAPS && a.taps.acc_ff2 && live[p])
-                        a.taps.acc_ff2[((bl[p] * KCF + cc) * T + t) * D + 32 * tile + ch(e, g)] = accbits(acc[p], e);
+                        a.taps.acc_ff2[((bl[p] * KCF + cc) * T + t) * D + 32 * tile + ch(e, g)] = accbits(acc[ai], e);
                 }
             };
 #pragma unroll
@@ -689,7 +703,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                 if constexpr (FP8) {
                     BF_DUO_PAIR_F8(false, 4 + HT * STEPS + cc, false, hid0 + 8 * cc * FRAG, hid0 + C::HID_P + 8 * cc * FRAG, acc);
 #pragma unroll
-                    for (int s = 0; s < 8; s++) { epi_2(cc, 0, s); epi_2(cc, 1, s); }
+                    for (int s = 0; s < 8; s++) { epi_2(cc, 0, s, 0); epi_2(cc, 1, s, 1); }
                 } else {
 #pragma unroll
                     for (int p = 0; p < NP; p++) {
@@ -703,15 +717,15 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                                 for (int k = 0; k < 4; k++) init[4 * j + k] = w0[j][k];
                         }
                         auto between = [&](int s) {
-                            if (n > 0) epi_2((n - 1) / NP, (n - 1) % NP, s);
+                            if (n > 0) epi_2((n - 1) / NP, (n - 1) % NP, s, (n - 1) & 1);
                         };
-                        BF_DUO_CHAIN(false, 4 + HT * STEPS + cc, p, hid0 + p * C::HID_P + 8 * cc * FRAG, init, acc[p], between);
+                        BF_DUO_CHAIN(false, 4 + HT * STEPS + cc, p, hid0 + p * C::HID_P + 8 * cc * FRAG, init, acc[n & 1], between);
                     }
                 }
             }
             if constexpr (!FP8)
 #pragma unroll
-                for (int s = 0; s < 8; s++) epi_2(KCF - 1, NP - 1, s);
+                for (int s = 0; s < 8; s++) epi_2(KCF - 1, NP - 1, s, (NP * KCF - 1) & 1);
             v4f b2[4];
             load_tile16(pB + C::B_BFF2 + 32 * sub, g, b2);
             const float sw = pB[C::B_SW + 16 + sub];
@@ -768,10 +782,13 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
     // Wave (m, p) multiplies head tile m (rows 32m..32m+31 of [policy; promo; value; 0]) with the
     // normalised stream of position p over the whole width, one fused-multiply-add chain in (tile,
     // quad, element) order; quarter 3's tile is zero and stores nothing, so it is not computed.
-    const int mine = sub;   // the position whose heads this wave computes
+    // With one position per workgroup the second wave of a quarter has nothing to do here but
+    // meet the barriers.
+    const int mine = NP == 2 ? sub : 0;   // the position whose heads this wave computes
+    const bool heads_here = NP == 2 || sub == 0;
     const float* const hnb = reinterpret_cast<const float*>(hid + mine * C::HID_P);
     v16f head = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    if (q < 3) {
+    if (q < 3 && heads_here) {
 #pragma unroll
         for (int hi = 0; hi < 2 * HB; hi++) {
             // the stream is padded by one block: two half-blocks past the last head block exist
@@ -786,9 +803,9 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         }
     }
     BF_PHASE(PH_HEADS);
-    const int b = mine ? bp[1] : bp[0];
-    const bool store = mine ? live[1] : live[0];
-    const int ctrl_m = mine ? ctrl[1] : ctrl[0];
+    const int b = mine ? bp[NP - 1] : bp[0];
+    const bool store = heads_here && (mine ? live[NP - 1] : live[0]);
+    const int ctrl_m = mine ? ctrl[NP - 1] : ctrl[0];
     auto value_of = [&](const v16f& hd) -> float {
         if (a.n_value == 1) return tanh_dev(hd[0]);
         const float r0 = hd[0], r1 = hd[1], r2 = hd[2];   // classes loss, draw, win
@@ -813,7 +830,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
     // policy (quarters 0 and 1: squares 0..31 and 32..63), optional legal-move AND and argmax
     float bv = -__builtin_inff();
     int bi = 0x7fffffff;
-    if (q < 2) {
+    if (q < 2 && heads_here) {
         unsigned long long mw = ~0ull;
         if (a.mask) mw = a.mask[(size_t)b * T + t];
 #pragma unroll
@@ -849,7 +866,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             bi = take ? oi : bi;
         }
         // the two policy waves' winners of a position meet in the exchange slot no row sum uses
-        if (q < 2 && lane == 0) {
+        if (q < 2 && heads_here && lane == 0) {
             xch[2 * XS + mine * 4 + q * 2] = bv;
             xch[2 * XS + mine * 4 + q * 2 + 1] = __int_as_float(bi);
         }
@@ -900,7 +917,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             }
         }
         barrier();
-        if (q == 2) {
+        if (q == 2 && heads_here) {
             // head tile 2 once more, against the pooled row (every token column holds the same row);
             // its blocks are read straight from the stream, in the same order as above
             v16f hd = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -927,21 +944,21 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
 #undef BF_PHASE
 }
 
-template <bool TAPS, bool FP8 = false, bool PROF = false>
+template <bool TAPS, bool FP8 = false, bool PROF = false, int NPOS = 2>
 hipError_t launch_duo(const KArgs& k, hipStream_t stream) {
     // more than 64 KiB of dynamic LDS has to be requested once per kernel and device
     static std::atomic<unsigned long long> lds_set{0};
-    constexpr int lds_bytes = Cfg<FP8>::LDS_BYTES;
+    constexpr int lds_bytes = Cfg<FP8, NPOS>::LDS_BYTES;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return hipErrorInvalidDevice;
     const unsigned long long bit = dev < 64 ? 1ull << dev : 0;
     if (!(lds_set.load(std::memory_order_relaxed) & bit)) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_kernel<TAPS, FP8, PROF>),
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&duo_kernel<TAPS, FP8, PROF, NPOS>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess) return e;
         lds_set.fetch_or(bit, std::memory_order_relaxed);
     }
-    hipLaunchKernelGGL((duo_kernel<TAPS, FP8, PROF>), dim3((k.n + 1) / 2), dim3(512), lds_bytes, stream, k);
+    hipLaunchKernelGGL((duo_kernel<TAPS, FP8, PROF, NPOS>), dim3((k.n + NPOS - 1) / NPOS), dim3(512), lds_bytes, stream, k);
     return hipGetLastError();
 }
 

@@ -224,14 +224,19 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream
     hipError_t e;
     if (!device_is_gfx950()) return BF_ERR_DEVICE;
     if (kind == BF_KERNEL_OCTO) {
-        if (k.profile)
-            e = a->shape.d_model == 512 ? bf::launch_octo512_prof(k, stream) : bf::launch_octo256_prof(k, stream);
+        // eight wavefronts per position: the 512-wide network and the e4m3 format on the board kernel's
+        // eight-wavefront form; the 256-wide int8 network on the two-position kernel's one-position
+        // form, which issues each product under the previous one's epilogue
+        if (k.profile && a->shape.d_model == 512)
+            e = bf::launch_octo512_prof(k, stream);
         else if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_octo512_taps(k, stream) : bf::launch_octo512(k, stream);
         else if (a->quant == BF_QUANT_E4M3)
             e = a->taps ? bf::launch_octo256_fp8_taps(k, stream) : bf::launch_octo256_fp8(k, stream);
+        else if (k.profile)
+            e = bf::launch_solo256_prof(k, stream);
         else
-            e = a->taps ? bf::launch_octo256_taps(k, stream) : bf::launch_octo256(k, stream);
+            e = a->taps ? bf::launch_solo256_taps(k, stream) : bf::launch_solo256(k, stream);
     } else if (kind == BF_KERNEL_DUO) {
         if (k.profile)
             e = bf::launch_duo256_prof(k, stream);

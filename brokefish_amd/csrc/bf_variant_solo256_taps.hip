@@ -1,0 +1,6 @@
+// Kernel variant "solo256_taps" of the evaluator (one position per workgroup of eight wavefronts, products issued under the previous epilogue), compiled as its own translation unit.
+#include "bf_duo.hip.h"
+
+namespace bf {
+hipError_t launch_solo256_taps(const KArgs& k, hipStream_t stream) { return duo::launch_duo<true, false, false, 1>(k, stream); }
+}  // namespace bf
