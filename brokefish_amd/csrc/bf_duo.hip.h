@@ -53,7 +53,11 @@ struct Cfg : Layout<256> {
     static constexpr int PAR_OFF = ACT_OFF + NP * ACT_P;
     static constexpr int PWL_FLOATS = A_FLOATS + B_FLOATS;
     static constexpr int TOK_OFF = PAR_OFF + 4 * PWL_FLOATS * 4;   // activation scale of every token, per position
-    static constexpr int LDS_BYTES = TOK_OFF + NP * 32 * 4;
+    static constexpr int USED_BYTES = TOK_OFF + NP * 32 * 4;
+    // The one-position form serves launches of at most one workgroup per compute unit: asking for
+    // more than half of a unit's LDS keeps the dispatcher from placing two of them on one unit
+    // while another unit stays empty.
+    static constexpr int LDS_BYTES = NP == 1 && USED_BYTES < 81 * 1024 ? 81 * 1024 : USED_BYTES;
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget: one workgroup per compute unit");
     static_assert(NT * 4 * FRAG <= HID_P, "normalised stream overlay");
 };
