@@ -28,12 +28,15 @@ HIP_SOURCES = ["bf_host.hip", "bf_expand.hip", "bf_movegen.hip", "bf_probe.hip",
                "bf_variant_twin256.hip", "bf_variant_twin256_taps.hip",
                "bf_variant_twin256_fp8.hip", "bf_variant_twin256_fp8_taps.hip",
                "bf_variant_board256_fp8.hip", "bf_variant_board256_fp8_taps.hip",
-                              "bf_variant_octo512.hip", "bf_variant_octo512_taps.hip",
+               "bf_variant_octo512.hip", "bf_variant_octo512_taps.hip",
                "bf_variant_octo256_fp8.hip", "bf_variant_octo256_fp8_taps.hip",
                "bf_variant_duo256.hip", "bf_variant_duo256_taps.hip",
                "bf_variant_duo256_fp8.hip", "bf_variant_duo256_fp8_taps.hip",
                "bf_variant_twin256_prof.hip", "bf_variant_duo256_prof.hip",
-               "bf_variant_solo256.hip", "bf_variant_solo256_taps.hip", "bf_variant_solo256_prof.hip", "bf_variant_octo512_prof.hip"]
+               "bf_variant_solo256.hip", "bf_variant_solo256_taps.hip", "bf_variant_solo256_prof.hip", "bf_variant_octo512_prof.hip",
+               "bf_variant_board256_prof.hip", "bf_variant_board512_prof.hip", "bf_variant_board256_fp8_prof.hip",
+               "bf_variant_twin256_fp8_prof.hip", "bf_variant_octo256_fp8_prof.hip", "bf_variant_duo256_fp8_prof.hip",
+               "bf_variant_prof_fp8.hip"]
 # -ffp-contract=off: the kernel's fp32 arithmetic is specified operation by operation
 # (fused multiply-adds are written explicitly), so the compiler must not fuse on its own.
 # The packed-fp32 feature is disabled so no v_pk_*_f32 instructions are generated.

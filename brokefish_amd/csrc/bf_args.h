@@ -157,10 +157,17 @@ hipError_t launch_duo256(const KArgs& k, hipStream_t stream);
 hipError_t launch_duo256_taps(const KArgs& k, hipStream_t stream);
 hipError_t launch_duo256_fp8(const KArgs& k, hipStream_t stream);
 hipError_t launch_duo256_fp8_taps(const KArgs& k, hipStream_t stream);
-// the int8 builds that carry the phase profile
+// the builds that carry the phase profile
 hipError_t launch_twin256_prof(const KArgs& k, hipStream_t stream);
 hipError_t launch_octo512_prof(const KArgs& k, hipStream_t stream);
 hipError_t launch_duo256_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_board256_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_board512_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_board256_fp8_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_twin256_fp8_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_octo256_fp8_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_duo256_fp8_prof(const KArgs& k, hipStream_t stream);
+hipError_t launch_prof_fp8(const KArgs& k, int grid, hipStream_t stream);
 // the same kernel with one position per workgroup (the eight-wavefront form for launches that
 // cannot fill the GPU): int8, 256-wide network
 hipError_t launch_solo256(const KArgs& k, hipStream_t stream);

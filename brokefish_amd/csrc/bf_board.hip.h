@@ -1112,6 +1112,12 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
                 for (int r = 0; r < 16; r++)
                     a.taps.resid[(bl * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = x[i][r];
     }
+    if (TAPS && a.taps.resid_last)
+#pragma unroll
+        for (int i = 0; i < TWW; i++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                a.taps.resid_last[((size_t)b * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = x[i][r];
 
     // ---- final norm and heads --------------------------------------------------------------------------
     // The first head block is in the fragment registers unless a layer range that stops early left

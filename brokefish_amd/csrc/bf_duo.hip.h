@@ -758,6 +758,13 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                     for (int r = 0; r < 16; r++)
                         a.taps.resid[(bl[p] * T + t) * D + 32 * tile + ch(r, g)] = x[p][r];
     }
+    if (TAPS && a.taps.resid_last)
+#pragma unroll
+        for (int p = 0; p < NP; p++)
+            if (live[p])
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    a.taps.resid_last[((size_t)bp[p] * T + t) * D + 32 * tile + ch(r, g)] = x[p][r];
 
     // ---- final norm and heads --------------------------------------------------------------------------
     // The weight stream is restarted at the head blocks (after the last layer the prefetch ran on

@@ -232,35 +232,42 @@ static int launch(const bf_eval_args* a, const bf::KArgs& k, int kind, hipStream
         else if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_octo512_taps(k, stream) : bf::launch_octo512(k, stream);
         else if (a->quant == BF_QUANT_E4M3)
-            e = a->taps ? bf::launch_octo256_fp8_taps(k, stream) : bf::launch_octo256_fp8(k, stream);
+            e = k.profile ? bf::launch_octo256_fp8_prof(k, stream)
+              : a->taps   ? bf::launch_octo256_fp8_taps(k, stream)
+                          : bf::launch_octo256_fp8(k, stream);
         else if (k.profile)
             e = bf::launch_solo256_prof(k, stream);
         else
             e = a->taps ? bf::launch_solo256_taps(k, stream) : bf::launch_solo256(k, stream);
     } else if (kind == BF_KERNEL_DUO) {
         if (k.profile)
-            e = bf::launch_duo256_prof(k, stream);
+            e = a->quant == BF_QUANT_E4M3 ? bf::launch_duo256_fp8_prof(k, stream) : bf::launch_duo256_prof(k, stream);
         else if (a->quant == BF_QUANT_E4M3)
             e = a->taps ? bf::launch_duo256_fp8_taps(k, stream) : bf::launch_duo256_fp8(k, stream);
         else
             e = a->taps ? bf::launch_duo256_taps(k, stream) : bf::launch_duo256(k, stream);
     } else if (kind == BF_KERNEL_TWIN) {
         if (k.profile)
-            e = bf::launch_twin256_prof(k, stream);
+            e = a->quant == BF_QUANT_E4M3 ? bf::launch_twin256_fp8_prof(k, stream) : bf::launch_twin256_prof(k, stream);
         else if (a->quant == BF_QUANT_E4M3)
             e = a->taps ? bf::launch_twin256_fp8_taps(k, stream) : bf::launch_twin256_fp8(k, stream);
         else
             e = a->taps ? bf::launch_twin256_taps(k, stream) : bf::launch_twin256(k, stream);
     } else if (kind == BF_KERNEL_BOARD) {
-        if (k.profile) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the TWIN, OCTO, DUO and QUAD kernels");
-        if (a->shape.d_model == 512)
+        if (k.profile)
+            e = a->shape.d_model == 512      ? bf::launch_board512_prof(k, stream)
+              : a->quant == BF_QUANT_E4M3 ? bf::launch_board256_fp8_prof(k, stream)
+                                          : bf::launch_board256_prof(k, stream);
+        else if (a->shape.d_model == 512)
             e = a->taps ? bf::launch_board512_taps(k, stream) : bf::launch_board512(k, stream);
         else if (a->quant == BF_QUANT_E4M3)
             e = a->taps ? bf::launch_board256_fp8_taps(k, stream) : bf::launch_board256_fp8(k, stream);
         else
             e = a->taps ? bf::launch_board256_taps(k, stream) : bf::launch_board256(k, stream);
     } else if (a->quant == BF_QUANT_E4M3)
-        e = a->taps ? bf::launch_taps_fp8(k, grid, stream) : bf::launch_prod_fp8(k, grid, stream);
+        e = k.profile ? bf::launch_prof_fp8(k, grid, stream)
+          : a->taps   ? bf::launch_taps_fp8(k, grid, stream)
+                      : bf::launch_prod_fp8(k, grid, stream);
     else
         e = k.profile ? bf::launch_prof(k, grid, stream)
           : a->taps   ? bf::launch_taps(k, grid, stream)
@@ -344,8 +351,6 @@ extern "C" int bf_profile_phases(const bf_eval_args* args, void* stream, uint64_
     const int rc = check_args(args, &k, &kind);
     if (rc) return rc;
     if (args->taps) return fail(BF_ERR_ARGUMENT, "the phase profile runs without taps");
-    if (args->quant != BF_QUANT_INT8) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the int8 format only");
-    if (kind == BF_KERNEL_BOARD) return fail(BF_ERR_UNSUPPORTED, "the phase profile is built for the TWIN, OCTO, DUO and QUAD kernels");
     if (!cycles) return fail(BF_ERR_ARGUMENT, "cycles must not be NULL");
     k.profile = reinterpret_cast<unsigned long long*>(cycles);
     return launch(args, k, kind, (hipStream_t)stream);

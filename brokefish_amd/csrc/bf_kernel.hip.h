@@ -551,6 +551,13 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
                     a.taps.resid[(bl * T + t) * D + 32 * n + ch(r, g)] = x[n][r];
         }
     }
+    if (TAPS && a.taps.resid_last && valid) {
+#pragma unroll
+        for (int n = 0; n < NT; n++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                a.taps.resid_last[((size_t)b * T + t) * D + 32 * n + ch(r, g)] = x[n][r];
+    }
 
     // ---- final norm and heads ------------------------------------------------------------------
     float hn[NT][16];

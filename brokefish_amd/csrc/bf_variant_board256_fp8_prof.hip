@@ -1,0 +1,6 @@
+// Kernel variant "board256_fp8_prof" of the evaluator (one position per workgroup, e4m3, with the phase profile), compiled as its own translation unit.
+#include "bf_board.hip.h"
+
+namespace bf {
+hipError_t launch_board256_fp8_prof(const KArgs& k, hipStream_t stream) { return board::launch_board<256, false, false, true, false, true>(k, stream); }
+}  // namespace bf

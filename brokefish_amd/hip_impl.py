@@ -43,7 +43,10 @@ class _Shape(C.Structure):
 
 
 _TAP_PTRS = ["embed", "qa_qkv", "acc_qkv", "qa_out", "acc_out", "qa_ff1", "acc_ff1",
-             "qa_ff2", "acc_ff2", "resid", "normed"]
+             "qa_ff2", "acc_ff2", "resid", "normed", "resid_last"]
+
+
+ABI_VERSION = 5     # BF_ABI_VERSION of include/brokefish_hip.h that the structs below mirror
 
 
 class _Taps(C.Structure):
@@ -125,6 +128,9 @@ def load_library():
         L.bf_abi_tag.restype = C.c_uint64
         # the ctypes mirror of bf_eval_args must be the struct the library was compiled with: a
         # shorter one would make the library read pointers from beyond it
+        if (L.bf_abi_tag() >> 32) != ABI_VERSION:
+            raise RuntimeError(f"{path} carries interface version {L.bf_abi_tag() >> 32}, this binding is written for "
+                               f"{ABI_VERSION}: rebuild the library (`__graft_entry__.build()`)")
         if (L.bf_abi_tag() & 0xFFFFFFFF) != C.sizeof(_Args):
             raise RuntimeError(f"{path} was built with a bf_eval_args of {L.bf_abi_tag() & 0xFFFFFFFF} bytes, this binding "
                                f"passes {C.sizeof(_Args)}: rebuild the library (`__graft_entry__.build()`)")
@@ -691,6 +697,8 @@ class FusedEncoder:
             self.board_wstream = torch.from_numpy(wstream).to(self.device)
             self.board_fparams = torch.from_numpy(fparams).to(self.device)
         self._buffered_full = 0
+        self._backbone = None
+        self._profile, self._profile_waves, self._profile_kept = None, 0, None
         self.best_move = None
 
     @property
@@ -822,24 +830,59 @@ class FusedEncoder:
             raise ValueError(f"expected [n, {T}, {self.d_model}], got {tuple(x.shape)}")
         if not x.is_cuda:
             raise ValueError("x must be on the GPU")
-        if alive is None:
-            alive_b = torch.ones(n, t, dtype=torch.bool, device=x.device)
-        else:
+        if alive is not None:
             if alive.shape != (n, t):
                 raise ValueError(f"alive must be [{n}, {t}], got {tuple(alive.shape)}")
             if alive.dtype not in (torch.bool, torch.int8):
                 raise ValueError(f"alive must be bool or int8, got {alive.dtype}")
-            alive_b = alive.bool()
-        # a captured slot is the word 0x800; only that bit reaches the attention mask here
-        boards = torch.where(alive_b, 0, 0x800).to(torch.int16)
-        control = torch.ones(n, dtype=torch.int16, device=x.device)
-        rep = torch.zeros(n, dtype=torch.uint8, device=x.device)
-        res = self.forward_taps(boards, control, rep, x_in=x.float().contiguous(), want=["resid"])
-        y = res["resid"][:, -1].to(x.dtype)
-        if out is not None:
-            out.copy_(y)
+        if out is not None and (out.shape != x.shape or out.device != x.device):
+            raise ValueError(f"out must be {tuple(x.shape)} on {x.device}")
+        # Everything the launch needs beyond x and out lives in buffers kept between calls, so a
+        # repeated call with out= given (fp32, contiguous) allocates nothing.
+        bb = self._backbone
+        if bb is None or bb["cap"] < n:
+            dev = self.device
+            bb = self._backbone = {
+                "cap": n, "boards": torch.zeros(n, T, dtype=torch.int16, device=dev),
+                "dead": torch.zeros(n, T, dtype=torch.bool, device=dev),
+                "control": torch.ones(n, dtype=torch.int16, device=dev),
+                "rep": torch.zeros(n, dtype=torch.uint8, device=dev),
+                "policy": torch.empty(n, T, N_POLICY, dtype=torch.float16, device=dev),
+                "promo": torch.empty(n, T, N_PROMO, dtype=torch.float16, device=dev),
+                "value": torch.empty(n, dtype=torch.float32, device=dev), "x": None, "y": None}
+        boards = bb["boards"][:n]
+        if alive is None:
+            boards.zero_()
+        else:
+            # a captured slot is the word 0x800; only that bit reaches the attention mask here
+            torch.logical_not(alive, out=bb["dead"][:n])
+            torch.mul(bb["dead"][:n], 0x800, out=boards)
+        if x.dtype is torch.float32 and x.is_contiguous():
+            x32 = x
+        else:
+            if bb["x"] is None or bb["x"].shape[0] < n:
+                bb["x"] = torch.empty(bb["cap"], T, d, dtype=torch.float32, device=self.device)
+            x32 = bb["x"][:n]
+            x32.copy_(x)
+        direct = out is not None and out.dtype is torch.float32 and out.is_contiguous()
+        if direct:
+            y32 = out
+        else:
+            if bb["y"] is None or bb["y"].shape[0] < n:
+                bb["y"] = torch.empty(bb["cap"], T, d, dtype=torch.float32, device=self.device)
+            y32 = bb["y"][:n]
+        taps = _Taps()
+        taps.x_in, taps.resid_last = x32.data_ptr(), y32.data_ptr()
+        taps.layer_begin, taps.layer_end = 0, self.n_layers
+        # the library copies the tap table at launch; the buffers it names stay alive in the cache
+        self._call(self._args(boards, bb["control"][:n], bb["rep"][:n], None, bb["policy"][:n], bb["promo"][:n],
+                              bb["value"][:n], None, taps))
+        if direct:
             return out
-        return y
+        if out is not None:
+            out.copy_(y32)
+            return out
+        return y32.to(x.dtype, copy=True)
 
     __call__ = forward
 
@@ -867,7 +910,18 @@ class FusedEncoder:
             if active is not None:
                 raise ValueError("a compacted leaf list replaces the active flags: pass one of them")
             leaves = _check_leaves(leaves, n, self.device)
-        if self.binding == "torch":
+        if self._profile is not None:
+            # set_profile(True): the launch goes through the phase-accounting build, which adds
+            # into the counters that read_profile returns
+            args = self._args(boards, control, rep, mask, self.policy_out, self.promo_out,
+                              self.value_out, self.best_out, active=active, leaves=leaves)
+            with torch.cuda.device(self.device):
+                rc = self._lib.bf_profile_phases(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
+                                                 C.c_void_p(self._profile.data_ptr()))
+            if rc:
+                raise RuntimeError(f"bf_profile_phases failed ({rc}): {self._lib.bf_last_error().decode()}")
+            self._profile_waves += self._launch_waves(n)
+        elif self.binding == "torch":
             for name, t in (("boards", boards), ("control", control), ("rep", rep), ("mask", mask), ("active", active)):
                 if t is not None and t.device != self.device:
                     raise ValueError(f"{name} is on {t.device}, the evaluator's weights are on {self.device}")
@@ -910,31 +964,60 @@ class FusedEncoder:
             raise RuntimeError(f"bf_time_kernel_ms failed ({ms}): {self._lib.bf_last_error().decode()}")
         return ms
 
+    def _launch_waves(self, n: int) -> int:
+        """Wavefronts in a launch of ``n`` positions of the kernel such a call runs."""
+        kind = self.kernel_choice(n)
+        return {"board": 4 * n, "twin": 4 * n, "octo": 8 * n, "duo": 8 * ((n + 1) // 2), "quad": 4 * ((n + 3) // 4)}[kind]
+
+    def profile_phase_names(self):
+        """Names of the counters of :meth:`read_profile`, in order (reference csrc/encoder.cu:1910)."""
+        return [self._lib.bf_profile_phase_name(i).decode() for i in range(self._lib.bf_profile_phase_count())]
+
+    def set_profile(self, on: bool) -> None:
+        """Phase accounting on or off for the ``forward_full`` calls that follow (reference
+        csrc/encoder.cu:1886, 1907): while on, each call runs the phase-accounting build of the
+        kernel it would run anyway (same outputs) and adds its shader-clock cycles per phase to the
+        counters.  Turning it on keeps counters already collected; ``reset_profile`` zeroes them."""
+        if on and self._profile is None:
+            self._profile = torch.zeros(self._lib.bf_profile_phase_count(), dtype=torch.int64, device=self.device)
+            self._profile_waves = 0
+        elif not on and self._profile is not None:
+            self._profile_kept = (self._profile, self._profile_waves)
+            self._profile = None
+
+    def reset_profile(self) -> None:
+        """Zero the cycle counters (reference csrc/encoder.cu:1888, 1908)."""
+        self._profile_kept = None
+        if self._profile is not None:
+            self._profile.zero_()
+            self._profile_waves = 0
+
+    def read_profile(self):
+        """``(cycles, wavefronts)``: the [phases] int64 cycle counters summed over all wavefronts
+        of the profiled launches since the last reset, and how many wavefronts that was (reference
+        csrc/encoder.cu:1894, 1909 returns the all-warps sum and warp 0's; here the sum and the
+        divisor).  Synchronises with the evaluator's stream."""
+        cyc, waves = (self._profile, self._profile_waves) if self._profile is not None else \
+            (self._profile_kept or (torch.zeros(self._lib.bf_profile_phase_count(), dtype=torch.int64), 0))
+        if cyc.is_cuda:
+            torch.cuda.current_stream(self.device).synchronize()
+        return cyc.cpu(), waves
+
     def profile_phases(self, boards, control, rep, mask=None) -> Dict[str, float]:
         """Shader-clock cycles per phase, averaged over the wavefronts of one launch of the
-        profiling build of the kernel this call would run (TWIN, OCTO, DUO or QUAD, int8): the
-        counterpart of the reference's read_profile / profile_phases.  ``sync_wait`` (time at
-        workgroup barriers) is also contained in the phases around it; ``total`` is a wavefront's
-        lifetime.  The outputs it writes are the normal ones."""
-        n = self._check_inputs(boards, control, rep, mask)
-        kind = self.kernel_choice(n)
-        if self.fp8 or kind == "board":
-            raise NotImplementedError("the phase profile is built for the int8 format on the TWIN, OCTO, DUO and QUAD "
-                                      "kernels (kernel='auto', 'twin', 'octo', 'duo' or 'quad')")
-        self._ensure_full_buffers(n)
-        k = self._lib.bf_profile_phase_count()
-        cyc = torch.zeros(k, dtype=torch.int64, device=self.device)
-        args = self._args(boards.contiguous(), control.contiguous(), rep.contiguous(),
-                          mask.contiguous() if mask is not None else None,
-                          self.policy_out, self.promo_out, self.value_out, self.best_out)
-        with torch.cuda.device(self.device):
-            rc = self._lib.bf_profile_phases(C.byref(args), C.c_void_p(torch.cuda.current_stream(self.device).cuda_stream),
-                                             C.c_void_p(cyc.data_ptr()))
-        if rc:
-            raise RuntimeError(f"bf_profile_phases failed ({rc}): {self._lib.bf_last_error().decode()}")
-        torch.cuda.current_stream(self.device).synchronize()
-        waves = {"twin": 4 * n, "octo": 8 * n, "duo": 8 * ((n + 1) // 2), "quad": 4 * ((n + 3) // 4)}[kind]
-        return {self._lib.bf_profile_phase_name(i).decode(): cyc[i].item() / waves for i in range(k)}
+        profiling build of the kernel this call would run: ``set_profile`` / one call /
+        ``read_profile`` in one step.  ``sync_wait`` (time at workgroup barriers) is also
+        contained in the phases around it; ``total`` is a wavefront's lifetime.  The outputs it
+        writes are the normal ones."""
+        saved = (self._profile, self._profile_waves, self._profile_kept)
+        self._profile = None
+        self.set_profile(True)
+        try:
+            self.forward_full(boards, control, rep, mask)
+            cyc, waves = self.read_profile()
+        finally:
+            self._profile, self._profile_waves, self._profile_kept = saved
+        return {name: cyc[i].item() / waves for i, name in enumerate(self.profile_phase_names())}
 
     # -- debug taps (the counterpart of the reference's forward_stage) ------------
 
@@ -973,7 +1056,8 @@ class FusedEncoder:
                   "qa_out": ((n, lr, T, d), torch.int8), "acc_out": ((n, lr, kd, T, d), torch.int32),
                   "qa_ff1": ((n, lr, T, d), torch.int8), "acc_ff1": ((n, lr, kd, T, f), torch.int32),
                   "qa_ff2": ((n, lr, T, f), torch.uint8), "acc_ff2": ((n, lr, kf, T, d), torch.int32),
-                  "resid": ((n, lr, T, d), torch.float32), "normed": ((n, T, d), torch.float32)}
+                  "resid": ((n, lr, T, d), torch.float32), "normed": ((n, T, d), torch.float32),
+                  "resid_last": ((n, T, d), torch.float32)}
         want = list(shapes) if want is None else list(want)
         out = {k: torch.zeros(shapes[k][0], dtype=shapes[k][1], device=dev) for k in want}
         taps = _Taps()

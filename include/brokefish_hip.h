@@ -41,8 +41,8 @@ enum bf_quant {
 };
 
 /* Five kernels compute the same function.
- *   QUAD   four positions per workgroup, one wavefront each, weights shared through LDS; carries
- *          the phase profile (256-wide network, int8 and e4m3).
+ *   QUAD   four positions per workgroup, one wavefront each, weights shared through LDS
+ *          (256-wide network, int8 and e4m3).
  *   BOARD  one position per workgroup, the four wavefronts split the model width; one workgroup
  *          per compute unit: low latency per position (launches that cannot fill the GPU);
  *          both network widths.
@@ -122,6 +122,9 @@ typedef struct {
     int32_t* acc_ff2;   /* [B,L,kc,32,d] accumulators of the unsigned product      */
     float* resid;       /* [B,L,32,d] residual stream after each layer             */
     float* normed;      /* [B,32,d]   after the final LayerNorm                    */
+    float* resid_last;  /* [B,32,d]   residual stream after the last layer run: what the
+                         * reference's encoder-only call returns
+                         * (brokefish/nn/cuda_impl.py:447-463) */
 } bf_taps;
 
 typedef struct {
@@ -193,7 +196,7 @@ typedef struct {
  * BF_ABI_TAG before its first call and refuses a library it was not built for (a shorter
  * bf_eval_args would make the library read pointers from beyond the caller's struct).  No
  * counterpart in the reference, whose module and kernels are one compilation. */
-#define BF_ABI_VERSION 4
+#define BF_ABI_VERSION 5
 #define BF_ABI_TAG (((uint64_t)BF_ABI_VERSION << 32) | (uint64_t)sizeof(bf_eval_args))
 uint64_t bf_abi_tag(void);
 
@@ -277,10 +280,12 @@ int bf_quant_probe(int mode, const float* x, float scale, int64_t n, uint8_t* ou
 /* In-kernel phase accounting, the counterpart of the reference's profile hooks
  * (reference csrc/encoder.cu:1083-1177 and :1886-1903: set_profile / read_profile /
  * profile_phases).  bf_profile_phases runs a separately compiled build of the kernel the
- * arguments select (TWIN, OCTO or QUAD; int8) that reads the shader clock at phase boundaries
- * and adds, per wavefront, the cycles of each phase into cycles[bf_profile_phase_count()]
- * (DEVICE memory, caller-zeroed): divide by the wavefronts of the launch (TWIN 4 n, OCTO 8 n,
- * QUAD 4 ceil(n / 4)).  Slot "sync_wait" is the time spent waiting at workgroup barriers (QUAD:
+ * arguments select (every kernel, both formats, both widths) that reads the shader clock at
+ * phase boundaries and ADDS, per wavefront, the cycles of each phase into
+ * cycles[bf_profile_phase_count()] (DEVICE memory, zeroed by the caller before the first launch
+ * it wants counted: several launches accumulate, as the reference's set_profile / read_profile
+ * pair does): divide by the wavefronts of the launches (BOARD and TWIN 4 n, OCTO 8 n, DUO
+ * 8 ceil(n / 2), QUAD 4 ceil(n / 4)).  Slot "sync_wait" is the time spent waiting at workgroup barriers (QUAD:
  * at the synchronisations of the LDS weight ring) and is also contained in the enclosing phases;
  * slot "total" is the wavefront lifetime.  In the one-position-per-workgroup kernels the matrix
  * products of a head are issued inside "qkv_gemm_epilogue" and those of the out-projection and

@@ -474,11 +474,13 @@ def test_weight_stream_probe_reports_a_plausible_rate():
     assert 8.0 < small < 45.0 and 2.0 < large < small, (small, large)
 
 
-@pytest.mark.parametrize("kernel,n", [("auto", 64), ("auto", 1000), ("quad", 64)])
-def test_phase_profile_runs_on_the_kernel_the_call_selects_and_leaves_the_outputs_right(kernel, n):
+@pytest.mark.parametrize("kernel,n,fmt", [("auto", 64, "int8"), ("auto", 1000, "int8"), ("quad", 64, "int8"), ("board", 40, "int8"),
+                                          ("twin", 300, "e4m3"), ("duo", 301, "e4m3"), ("octo", 33, "e4m3"), ("board", 20, "e4m3"),
+                                          ("quad", 30, "e4m3")])
+def test_phase_profile_runs_on_the_kernel_the_call_selects_and_leaves_the_outputs_right(kernel, n, fmt):
     torch.manual_seed(0)
     net = BrokefishNet().eval()
-    model = encoder_impl("hip")(net, int8=True, kernel=kernel)
+    model = encoder_impl("hip")(net, int8=fmt == "int8", fp8=fmt == "e4m3", kernel=kernel)
     b, c, r, m = positions.random_positions(n, plies=120, seed=5)
     bd, cd, rd, md = (t.cuda() for t in (b, c, r, m))
     want = [t.clone() for t in model.forward_full(bd, cd, rd, md)]
@@ -491,5 +493,50 @@ def test_phase_profile_runs_on_the_kernel_the_call_selects_and_leaves_the_output
     assert 0.9 * ph["total"] <= parts <= 1.0001 * ph["total"], ph   # the phases tile the wavefront's life
     for got, w in zip((model.policy_out, model.promo_out, model.value_out), want):
         assert torch.equal(got, w)
-    with pytest.raises(NotImplementedError):
-        encoder_impl("hip")(net, int8=True, kernel="board").profile_phases(bd, cd, rd, md)
+
+
+def test_phase_profile_of_the_512_wide_network_on_both_of_its_kernels():
+    torch.manual_seed(0)
+    net = BrokefishNet(d_model=512, n_heads=16, d_ff=2048, n_layers=2).eval()
+    b, c, r, m = positions.random_positions(24, plies=120, seed=6)
+    bd, cd, rd, md = (t.cuda() for t in (b, c, r, m))
+    for kernel in ("board", "octo"):
+        model = encoder_impl("hip")(net, int8=True, kernel=kernel)
+        want = [t.clone() for t in model.forward_full(bd, cd, rd, md)]
+        ph = model.profile_phases(bd, cd, rd, md)
+        parts = sum(v for k, v in ph.items() if k not in ("sync_wait", "total"))
+        assert ph["total"] > 0 and 0.9 * ph["total"] <= parts <= 1.0001 * ph["total"], (kernel, ph)
+        for got, w in zip((model.policy_out, model.promo_out, model.value_out), want):
+            assert torch.equal(got, w)
+
+
+def test_set_profile_accumulates_over_calls_until_reset_like_the_references_switch():
+    """reference csrc/encoder.cu:1886-1903 and bench/bench_phases.py:99-105: set_profile(True),
+    reset_profile(), run, read_profile(), set_profile(False)."""
+    torch.manual_seed(0)
+    net = BrokefishNet().eval()
+    model = encoder_impl("hip")(net, int8=True)
+    b, c, r, m = positions.random_positions(600, plies=120, seed=7)
+    bd, cd, rd, md = (t.cuda() for t in (b, c, r, m))
+    want = [t.clone() for t in model.forward_full(bd, cd, rd, md)]
+    names = model.profile_phase_names()
+    assert names[-1] == "total" and "sync_wait" in names
+    cyc, waves = model.read_profile()
+    assert waves == 0 and int(cyc.sum()) == 0               # nothing recorded before it is switched on
+    model.set_profile(True)
+    model.reset_profile()
+    model.forward_full(bd, cd, rd, md)
+    one, w1 = model.read_profile()
+    assert w1 == 8 * 300 and int(one[-1]) > 0               # 600 positions on the two-position kernel
+    model.forward_full(bd, cd, rd, md)
+    model.forward_full(bd[:100], cd[:100], rd[:100], md[:100])       # a small call: eight wavefronts per position
+    two, w2 = model.read_profile()
+    assert w2 == 2 * w1 + 800 and (two >= one).all() and int(two[-1]) > 1.5 * int(one[-1])
+    model.set_profile(False)
+    kept, wk = model.read_profile()
+    assert wk == w2 and torch.equal(kept, two)              # switched off: the counters stay readable
+    got = model.forward_full(bd, cd, rd, md)                # and calls are no longer counted
+    assert all(torch.equal(g, w) for g, w in zip(got, want))
+    assert model.read_profile()[1] == w2
+    model.reset_profile()
+    assert model.read_profile()[1] == 0

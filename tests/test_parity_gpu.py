@@ -348,6 +348,37 @@ def test_backbone_call_from_a_bare_encoder_stack(nets):
     assert torch.equal(got2[alive.cuda()], got[alive.cuda()])
 
 
+def test_backbone_call_with_an_output_buffer_allocates_nothing_once_warm(nets):
+    # reference brokefish/nn/cuda_impl.py:447-463 takes out= so that a serving loop can reuse one
+    # buffer; here the whole call then runs out of buffers kept between calls
+    net, sd, model, co = nets["distinct"]
+    b, c, r, _ = positions.random_positions(700, plies=100, seed=18)
+    with torch.no_grad():
+        x, alive = emulated.embed(sd, b, c, r)
+    xd, ad = x.cuda(), alive.cuda()
+    out = torch.empty_like(xd)
+    want = model.forward(xd, ad).clone()                       # two positions per workgroup at this size
+    idx = np.arange(0, 700, 29)
+    ref = co.forward(b.numpy()[idx], c.numpy()[idx], r.numpy()[idx], taps=True)["resid"][:, -1]
+    assert _bits_equal(want[idx], ref)
+    model.forward(xd, ad, out=out)                             # warm: buffers exist from here on
+    torch.cuda.synchronize()
+    count = lambda: torch.cuda.memory_stats()["allocation.all.allocated"]
+    before = count()
+    out.zero_()
+    assert model.forward(xd, ad, out=out) is out
+    model.forward(xd[:40], ad[:40], out=out[:40])              # a smaller call reuses the same buffers
+    model.forward(xd[:40], None, out=out[:40])
+    assert count() == before
+    assert torch.equal(out[40:], want[40:])
+    everyone = model.forward(xd[:40], torch.ones_like(ad[:40]))
+    assert torch.equal(out[:40], everyone)
+    # a half-precision caller: converted through kept buffers, the result comes back in its dtype
+    oh = torch.empty(700, 32, 256, dtype=torch.float16, device="cuda")
+    model.forward(xd.half(), ad, out=oh)
+    assert torch.equal(oh, model.forward(xd.half().float(), ad).half())
+
+
 def test_full_batch_properties_at_4096(nets):
     # the metric's batch size: spot-check against the C checker, and size-independent properties
     net, sd, model, co = nets["seed0"]

@@ -16,7 +16,8 @@ def test_extension_module_loads_and_exports_the_reference_modules_functions():
     assert ext.profile_phase_names()[-1] == "total" and "attention" in ext.profile_phase_names()
     # AUTO: eight wavefronts per position up to one position per compute unit, the throughput kernel above
     assert ext.kernel_choice(256, 8, 8, 1024, 1, 64, 0, 0, True) == 4
-    assert ext.kernel_choice(256, 8, 8, 1024, 1, 4096, 0, 0, True) == 3
+    assert ext.kernel_choice(256, 8, 8, 1024, 1, 4096, 0, 0, True) == 5     # two positions per workgroup
+    assert ext.kernel_choice(256, 8, 8, 1024, 1, 4096, 1, 0, True) == 3     # e4m3: one position per workgroup, two workgroups per unit
     assert ext.kernel_choice(512, 16, 16, 2048, 1, 4096, 0, 0, True) == 4
     with pytest.raises(RuntimeError):
         ext.kernel_choice(384, 8, 12, 1536, 1, 64, 0, 0, True)
