@@ -71,7 +71,7 @@
 // they compile only together with BF_TIMING_BUILD, which the library's own build never defines
 // (brokefish_amd/_build.py refuses both).
 #if (defined(BF_EXP_NOF32) || defined(BF_EXP_NOMFMA) || defined(BF_EXP_SAMEBLOCK) || defined(BF_EXP_NOLOAD) || \
-     defined(BF_EXP_HALFLOAD) || defined(BF_EXP_NOBARRIER)) && !defined(BF_TIMING_BUILD)
+     defined(BF_EXP_HALFLOAD) || defined(BF_EXP_NOBARRIER) || defined(BF_EXP_SAMELAYER) || defined(BF_EXP_NOWARM)) && !defined(BF_TIMING_BUILD)
 #error "BF_EXP_* switches give wrong results: they need BF_TIMING_BUILD and never go into the library"
 #endif
 #ifdef BF_EXP_NOF32   // timing experiment: one vector instruction in place of an fp32 matrix step

@@ -191,6 +191,43 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         load_half(2 * ((n < NB ? base : next) + at.a + sub * at.b) + hh % 2, hh % NSETS);
     };
 
+    // L2 warm-up for launches of one wave of workgroups (NP == 1): such a launch moves through the
+    // layers in step, so every first touch of a weight line would be an L2 miss that all the
+    // workgroups behind that L2 wait for.  The workgroups of an XCD (dispatched round-robin, so
+    // blockIdx / 8 numbers them) each touch a share of the lines of a layer's blocks one layer ahead,
+    // one dword per 128-byte line; the values are never used.  A hint only: a share that nobody
+    // touches (workgroups that left early, another dispatch order) costs time, not correctness.
+    // Below four workgroups per XCD the touches cover too little to pay for the loads they delay
+    // (loads return in order), above one workgroup per compute unit the launch is not in step.
+#ifdef BF_EXP_NOWARM   // timing experiment: no warm-up touches (results stay right)
+    constexpr int WARM = 0;
+#else
+    constexpr int WARM = NP == 1 ? 2 : 0;
+#endif
+    constexpr int LAYER_LINES = BPW * BLOCK / 128;   // per quarter
+    int warm[WARM > 0 ? WARM : 1] = {};
+    auto warm_l2 = [&](int blk0) {
+        if constexpr (WARM > 0) {
+            const int per = ((int)gridDim.x + 7) >> 3;
+#pragma unroll
+            for (int j = 0; j < WARM; j++) {
+                const int line = ((j * per + ((int)blockIdx.x >> 3)) * 8 + wave) * 64 + lane;
+                if (line < 4 * LAYER_LINES && gridDim.x > 24 && gridDim.x <= 256) {
+                    const int qq = line / LAYER_LINES, off = line % LAYER_LINES;
+                    warm[j] = *reinterpret_cast<const int*>(
+                        a.wstream + ((size_t)qq * ((size_t)a.n_layers * BPW + HB + 1) + (size_t)blk0) * BLOCK + (size_t)off * 128);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto warm_done = [&]() {   // the touches have long returned: retire their registers
+        if constexpr (WARM > 0) {
+#pragma unroll
+            for (int j = 0; j < WARM; j++) asm volatile("" ::"v"(warm[j]));
+        }
+    };
+
     // Row sum over the width for both positions: a wave's 16 values form one chain from zero, the
     // two tile sums of a quarter are added, then the four quarter sums in order.  One exchange slot
     // per call site, so that a fast wave's next partial cannot overwrite what a slow wave still
@@ -291,7 +328,8 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
     // ---- start the weight stream and the first layer's parameters --------------------------------
     if (nl_run > 0) {
 #pragma unroll
-        for (int j = 0; j < NSETS - 1; j++) fetch_half(j, 0, BPW);
+        for (int j = 0; j < NSETS; j++) fetch_half(j, 0, BPW);
+        warm_l2(a.l0 * BPW);
         if (par_owner) {
             dma(wpar + (size_t)a.l0 * C::PW_FLOATS, pA, C::A_FLOATS, lane);
             dma(wpar + (size_t)a.l0 * C::PW_FLOATS + C::A_FLOATS, pB, C::B_FLOATS, lane);
@@ -350,6 +388,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
     }
 
     wait_vm<0>();   // the parameters have landed (published to the quarter's other wave by the next barrier)
+    warm_done();
     BF_PHASE(PH_EMBED);
 
     for (int l = a.l0; l < a.l1; l++) {
@@ -358,12 +397,17 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
 #pragma unroll
         for (int p = 0; p < NP; p++) bl[p] = (size_t)bp[p] * nl_run + li;
         const int lnext = l + 1 < a.l1 ? l + 1 : l;   // after the last layer the same layer is fetched again (and never used)
+#ifdef BF_EXP_SAMELAYER   // timing experiment: every layer streams the first layer's blocks (they stay in L2)
+        const int lbase = 0 * li, lfollow = 0 * lnext;
+#else
         const int lbase = li * BPW, lfollow = (lnext - a.l0) * BPW;
+#endif
         // One position's product with the wave's k-th block of this layer: eight 32-deep steps against
         // the operand row whose fragment 0 is at BSRC (lane offset included), each fragment fetched
         // from LDS one step ahead.  The block's two halves sit in register sets 2k % NSETS and
-        // (2k + 1) % NSETS; position 0 goes first and starts the fetch of the half-block NSETS - 1
-        // positions on, position 1 refills the first half's set once it has consumed it.
+        // (2k + 1) % NSETS; the last position refills each of them as soon as it has consumed it (with
+        // the half-blocks NSETS on), so every set is in flight or full across the phases between
+        // products (attention, the LayerNorms).
         // BETWEEN(s) runs after step s has been issued: an eighth of the previous product's epilogue,
         // which the vector ALU works through while the matrix pipe runs; nothing is scheduled across
         // the end of a step.
@@ -374,7 +418,6 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
     do {                                                                                             \
         constexpr int A_ = BF_DUO_AHEAD;                                                             \
         const uint8_t* const b_ = (BSRC);                                                            \
-        if ((p) == 0) fetch_half(2 * (k) + NSETS - 1, lbase, lfollow);                               \
         v4i ring_[A_ + 1];                                                                           \
         _Pragma("unroll") for (int u_ = 0; u_ < A_; u_++) ring_[u_] = ldsfrag(b_ + u_ * FRAG);       \
         (R) = (INIT);                                                                                \
@@ -385,6 +428,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             __builtin_amdgcn_sched_barrier(0);                                                       \
             if ((p) == NP - 1 && s_ == 3) fetch_half(2 * (k) + NSETS, lbase, lfollow);               \
         }                                                                                            \
+        if ((p) == NP - 1) fetch_half(2 * (k) + NSETS + 1, lbase, lfollow);                          \
     } while (0)
         // e4m3: both positions' products with the wave's k-th block, step by step.  A weight fragment is
         // widened to fp16 once and multiplied with both positions' operands; these come from LDS
@@ -393,7 +437,6 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
 #define BF_DUO_PAIR_F8(SWAP, k, A16, B0, B1, R)                                                      \
     do {                                                                                             \
         const uint8_t* const bp_[2] = {(B0), (B1)};                                                  \
-        fetch_half(2 * (k) + NSETS - 1, lbase, lfollow);                                             \
         (R)[0] = zero;                                                                               \
         (R)[1] = zero;                                                                               \
         /* the operands of a step are fetched from LDS one step ahead: [position][half] */           \
@@ -420,6 +463,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                 _Pragma("unroll") for (int h_ = 0; h_ < ((A16) ? 2 : 1); h_++) cur_[p_][h_] = nxt_[p_][h_]; \
             if (s_ == 3) fetch_half(2 * (k) + NSETS, lbase, lfollow);                                \
         }                                                                                            \
+        fetch_half(2 * (k) + NSETS + 1, lbase, lfollow);                                             \
     } while (0)
         const acc_t zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         auto none = [&](int) {};
@@ -511,6 +555,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
                 for (int s = 0; s < 8; s++) epi_v(NP - 1, s, (3 * NP - 1) & 1);
             }
             BF_PHASE(PH_QKV);
+            if (l + 1 < a.l1) warm_l2((l + 1) * BPW);   // the sets are full and the next weight wait is an attention away
 #pragma unroll
             for (int p = 0; p < NP; p++) {
                 // scores, transposed: lane = query token, register r = key ch(r, g)
@@ -748,6 +793,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
             }
         }
         BF_PHASE(PH_FF2);
+        warm_done();
 #undef BF_DUO_CHAIN
 #undef BF_DUO_PAIR_F8
         if (TAPS && a.taps.resid)
