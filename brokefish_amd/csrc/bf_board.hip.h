@@ -510,8 +510,12 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 
     // ---- embedding (this wave's channels) --------------------------------------------------------
     float x[TWW][16];
-    const unsigned word = a.boards[(size_t)b * T + t];
-    const int ctrl = a.control[b];
+    // An encoder-only launch (tap table with `alive`): the residual stream comes in through x_in, the
+    // token mask through `alive`, the stream after the last layer goes out through resid_last, and
+    // there are no board words and no heads.
+    const bool enc_only = TAPS && a.taps.alive != nullptr;
+    const unsigned word = enc_only ? (a.taps.alive[(size_t)b * T + t] ? 0u : 0x800u) : a.boards[(size_t)b * T + t];
+    const int ctrl = enc_only ? 1 : a.control[b];
     const unsigned alive = (unsigned)__ballot(((word >> 11) & 1) == 0 && g == 0);
     if (TAPS && a.taps.x_in) {
 #pragma unroll
@@ -1118,6 +1122,7 @@ __global__ __launch_bounds__(OCTO ? 2 * THREADS : THREADS, TWIN && !OCTO ? BF_TW
 #pragma unroll
             for (int r = 0; r < 16; r++)
                 a.taps.resid_last[((size_t)b * T + t) * D + 32 * (TW * q + t0 + i) + ch(r, g)] = x[i][r];
+    if (enc_only) return;   // the same for every wave of the launch
 
     // ---- final norm and heads --------------------------------------------------------------------------
     // The first head block is in the fragment registers unless a layer range that stops early left

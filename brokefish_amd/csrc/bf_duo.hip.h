@@ -336,6 +336,10 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
         }
     }
 
+    // An encoder-only launch (tap table with `alive`): the residual stream comes in through x_in, the
+    // token mask through `alive`, the stream after the last layer goes out through resid_last, and
+    // there are no board words and no heads.
+    const bool enc_only = TAPS && a.taps.alive != nullptr;
     // ---- embedding (this wave's tile, both positions) ----------------------------------------------
     float x[NP][16];
     unsigned alive[NP];
@@ -343,8 +347,8 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
 #pragma unroll
     for (int p = 0; p < NP; p++) {
         const int b = bp[p];
-        const unsigned word = a.boards[(size_t)b * T + t];
-        ctrl[p] = a.control[b];
+        const unsigned word = enc_only ? (a.taps.alive[(size_t)b * T + t] ? 0u : 0x800u) : a.boards[(size_t)b * T + t];
+        ctrl[p] = enc_only ? 1 : a.control[b];
         alive[p] = (unsigned)__ballot(((word >> 11) & 1) == 0 && g == 0);
         if (TAPS && a.taps.x_in) {
 #pragma unroll
@@ -811,6 +815,7 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                     a.taps.resid_last[((size_t)bp[p] * T + t) * D + 32 * tile + ch(r, g)] = x[p][r];
+    if (enc_only) return;   // the same for every wave of the launch
 
     // ---- final norm and heads --------------------------------------------------------------------------
     // The weight stream is restarted at the head blocks (after the last layer the prefetch ran on

@@ -150,18 +150,28 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
     if (*kind < 0) return *kind;
     const bool board = *kind == BF_KERNEL_BOARD || *kind == BF_KERNEL_TWIN || *kind == BF_KERNEL_OCTO || *kind == BF_KERNEL_DUO;
     if (a->n < 1 || a->n > (1ll << 28)) return fail(BF_ERR_ARGUMENT, "n must be in [1, 2^28]");
-    if (!a->boards || !a->control || !a->rep) return fail(BF_ERR_ARGUMENT, "boards/control/rep must not be NULL");
-    if (!a->policy || !a->promo || !a->value) return fail(BF_ERR_ARGUMENT, "policy/promo/value must not be NULL");
+    // encoder-only launch: residual stream in and out through the tap table, no board words, no heads
+    const bool enc_only = a->taps && a->taps->alive;
+    if (enc_only) {
+        if (!a->taps->x_in || !a->taps->resid_last)
+            return fail(BF_ERR_ARGUMENT, "an encoder-only launch (taps.alive) needs taps.x_in and taps.resid_last");
+        if ((uintptr_t)a->taps->resid_last & 15) return fail(BF_ERR_ARGUMENT, "resid_last must be 16-byte aligned");
+        if (a->leaf_index || a->leaf_count || a->active)
+            return fail(BF_ERR_ARGUMENT, "an encoder-only launch takes neither active flags nor a leaf list");
+    } else {
+        if (!a->boards || !a->control || !a->rep) return fail(BF_ERR_ARGUMENT, "boards/control/rep must not be NULL");
+        if (!a->policy || !a->promo || !a->value) return fail(BF_ERR_ARGUMENT, "policy/promo/value must not be NULL");
+    }
     const uint8_t* ws = board ? a->board_wstream : a->wstream;
     const float* fp = board ? a->board_fparams : a->fparams;
     if (((uintptr_t)ws & 15) || ((uintptr_t)fp & 15))
         return fail(BF_ERR_ARGUMENT, "the parameter blobs must be 16-byte aligned");
-    if (((uintptr_t)a->policy & 15) || ((uintptr_t)a->promo & 7))
+    if (!enc_only && (((uintptr_t)a->policy & 15) || ((uintptr_t)a->promo & 7)))
         return fail(BF_ERR_ARGUMENT, "policy must be 16-byte and promo 8-byte aligned");
-    if (((uintptr_t)a->boards & 1) || ((uintptr_t)a->control & 1) || ((uintptr_t)a->value & 3) ||
-        ((uintptr_t)a->mask & 7) || ((uintptr_t)a->best_move & 3))
+    if (!enc_only && (((uintptr_t)a->boards & 1) || ((uintptr_t)a->control & 1) || ((uintptr_t)a->value & 3) ||
+                      ((uintptr_t)a->mask & 7) || ((uintptr_t)a->best_move & 3)))
         return fail(BF_ERR_ARGUMENT, "boards/control/value/mask/best_move must be aligned to their element size");
-    if (a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
+    if (!enc_only && a->best_move && !a->mask) return fail(BF_ERR_ARGUMENT, "best_move needs a mask");
     if ((a->leaf_index == nullptr) != (a->leaf_count == nullptr))
         return fail(BF_ERR_ARGUMENT, "leaf_index and leaf_count come together");
     if (a->leaf_index && a->active) return fail(BF_ERR_ARGUMENT, "a compacted leaf list replaces the active flags: pass one of them");
@@ -192,6 +202,10 @@ static int check_args(const bf_eval_args* a, bf::KArgs* k, int* kind) {
                 return fail(BF_ERR_ARGUMENT, "taps layer range must satisfy 0 <= begin <= end <= n_layers");
         }
         if (a->taps->x_in && ((uintptr_t)a->taps->x_in & 15)) return fail(BF_ERR_ARGUMENT, "x_in must be 16-byte aligned");
+    }
+    if (enc_only) {   // nothing of these is read or written
+        k->boards = nullptr; k->control = nullptr; k->rep = nullptr; k->mask = nullptr;
+        k->policy = nullptr; k->promo = nullptr; k->value = nullptr; k->best = nullptr;
     }
     return BF_OK;
 }

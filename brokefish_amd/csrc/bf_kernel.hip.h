@@ -183,8 +183,12 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
 
     // ---- embedding ---------------------------------------------------------------------
     float x[NT][16];
-    const unsigned word = a.boards[(size_t)b * T + t];
-    const int ctrl = a.control[b];
+    // An encoder-only launch (tap table with `alive`): the residual stream comes in through x_in, the
+    // token mask through `alive`, the stream after the last layer goes out through resid_last, and
+    // there are no board words and no heads.
+    const bool enc_only = TAPS && a.taps.alive != nullptr;
+    const unsigned word = enc_only ? (a.taps.alive[(size_t)b * T + t] ? 0u : 0x800u) : a.boards[(size_t)b * T + t];
+    const int ctrl = enc_only ? 1 : a.control[b];
     const unsigned alive = (unsigned)__ballot(((word >> 11) & 1) == 0 && g == 0);
     if (TAPS && a.taps.x_in) {
 #pragma unroll
@@ -558,6 +562,7 @@ __global__ __launch_bounds__(THREADS, 1) void eval_kernel(const KArgs a) {
             for (int r = 0; r < 16; r++)
                 a.taps.resid_last[((size_t)b * T + t) * D + 32 * n + ch(r, g)] = x[n][r];
     }
+    if (enc_only) return;   // the same for every wave of the launch
 
     // ---- final norm and heads ------------------------------------------------------------------
     float hn[NT][16];

@@ -125,6 +125,55 @@ void model_forward(torch::Tensor boards, torch::Tensor control, torch::Tensor re
     TORCH_CHECK(rc == BF_OK, "bf_model_forward failed (", rc, "): ", bf_last_error());
 }
 
+// The encoder stack alone, in place on y (reference csrc/encoder.cu:1752-1764 encoder_forward(y,
+// weights, alive, n_layers, eps, debug_stage)): y [n, 32, d_model] float32 is the residual stream
+// entering the first layer and, on return, the stream leaving the last; alive [n, 32] int8 or bool
+// masks dead tokens out of attention as keys.  No heads run and nothing is allocated.
+void encoder_forward(torch::Tensor y, torch::Tensor weights, torch::Tensor params, torch::Tensor alive,
+                     int64_t d_model, int64_t n_layers, int64_t n_heads, int64_t d_ff, double eps, int64_t quant,
+                     int64_t kernel, int64_t n_value, OptTensor workspace_) {
+    const torch::Tensor workspace = get(workspace_);
+    TORCH_CHECK(y.is_cuda() && y.scalar_type() == torch::kFloat && y.is_contiguous() && y.dim() == 3 &&
+                    y.size(1) == BF_TOKENS && y.size(2) == d_model && y.size(0) >= 1,
+                "y must be [n, 32, d_model] float32 contiguous on the GPU");
+    const auto dev = y.device();
+    auto on_dev = [&](const torch::Tensor& t) { return t.is_cuda() && t.device() == dev && t.is_contiguous(); };
+    TORCH_CHECK(on_dev(alive) && (alive.scalar_type() == torch::kChar || alive.scalar_type() == torch::kBool) &&
+                    alive.numel() == y.size(0) * BF_TOKENS,
+                "alive must be [n, 32] int8 or bool on y's device");
+    TORCH_CHECK(on_dev(weights) && weights.scalar_type() == torch::kByte, "weights must be a uint8 blob on y's device");
+    TORCH_CHECK(on_dev(params) && params.scalar_type() == torch::kFloat, "params must be a float32 blob on y's device");
+    bf_eval_args a{};
+    bf_taps taps{};
+    a.n = y.size(0);
+    a.shape = bf_shape{(int32_t)d_model, (int32_t)n_layers, (int32_t)n_heads, (int32_t)d_ff, (int32_t)n_value, (float)eps};
+    if (kernel == BF_KERNEL_QUAD) {
+        a.wstream = static_cast<const uint8_t*>(weights.data_ptr());
+        a.fparams = static_cast<const float*>(params.data_ptr());
+        TORCH_CHECK((size_t)weights.numel() == bf_wstream_bytes(&a.shape) && (size_t)params.numel() == bf_fparams_floats(&a.shape),
+                    "weights / params are not the blobs of this shape for the four-positions-per-workgroup kernel");
+        TORCH_CHECK(!absent(workspace) && on_dev(workspace) && (size_t)workspace.numel() >= bf_workspace_bytes(&a.shape, a.n),
+                    "the four-positions-per-workgroup kernel needs a workspace of bf_workspace_bytes(shape, n) bytes");
+        a.workspace = workspace.data_ptr();
+        a.workspace_bytes = (size_t)workspace.numel();
+    } else {
+        a.board_wstream = static_cast<const uint8_t*>(weights.data_ptr());
+        a.board_fparams = static_cast<const float*>(params.data_ptr());
+        TORCH_CHECK((size_t)weights.numel() == bf_board_wstream_bytes(&a.shape) &&
+                        (size_t)params.numel() == bf_board_fparams_floats(&a.shape),
+                    "weights / params are not the blobs of this shape for the one-position-per-workgroup kernels");
+    }
+    a.quant = (int32_t)quant;
+    a.kernel = (int32_t)kernel;
+    taps.x_in = static_cast<const float*>(y.data_ptr());
+    taps.resid_last = static_cast<float*>(y.data_ptr());
+    taps.alive = static_cast<const int8_t*>(alive.data_ptr());
+    a.taps = &taps;   // copied by the library before the call returns
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(dev);
+    const int rc = bf_model_forward(&a, c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(dev.index()).stream());
+    TORCH_CHECK(rc == BF_OK, "bf_model_forward failed (", rc, "): ", bf_last_error());
+}
+
 // Cycles per phase summed over the wavefronts of one launch of the profiling build (see
 // bf_profile_phases); returns an int64 tensor on the device, already written when it is read.
 torch::Tensor profile_phases(torch::Tensor boards, torch::Tensor control, torch::Tensor rep, torch::Tensor weights,
@@ -151,6 +200,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("quant") = 0, py::arg("kernel") = 0, py::arg("n_value") = 1, py::arg("vmode") = 0,
           py::arg("mask") = py::none(), py::arg("best_move") = py::none(), py::arg("active") = py::none(),
           py::arg("workspace") = py::none(), py::arg("leaf_index") = py::none(), py::arg("leaf_count") = py::none());
+    m.def("encoder_forward", &encoder_forward, "the encoder stack alone, in place on y", py::arg("y"), py::arg("weights"),
+          py::arg("params"), py::arg("alive"), py::arg("d_model"), py::arg("n_layers"), py::arg("n_heads"), py::arg("d_ff"),
+          py::arg("eps"), py::arg("quant") = 0, py::arg("kernel") = 0, py::arg("n_value") = 1, py::arg("workspace") = py::none());
     m.def("profile_phases", &profile_phases, "cycles per phase of one profiled launch", py::arg("boards"),
           py::arg("control"), py::arg("rep"), py::arg("weights"), py::arg("params"), py::arg("policy"), py::arg("promo"),
           py::arg("value"), py::arg("d_model"), py::arg("n_layers"), py::arg("n_heads"), py::arg("d_ff"), py::arg("eps"),

@@ -46,12 +46,12 @@ _TAP_PTRS = ["embed", "qa_qkv", "acc_qkv", "qa_out", "acc_out", "qa_ff1", "acc_f
              "qa_ff2", "acc_ff2", "resid", "normed", "resid_last"]
 
 
-ABI_VERSION = 5     # BF_ABI_VERSION of include/brokefish_hip.h that the structs below mirror
+ABI_VERSION = 6     # BF_ABI_VERSION of include/brokefish_hip.h that the structs below mirror
 
 
 class _Taps(C.Structure):
     _fields_ = ([("x_in", C.c_void_p), ("layer_begin", C.c_int32), ("layer_end", C.c_int32)]
-                + [(n, C.c_void_p) for n in _TAP_PTRS])
+                + [(n, C.c_void_p) for n in _TAP_PTRS] + [("alive", C.c_void_p)])
 
 
 class _ExpandArgs(C.Structure):
@@ -837,26 +837,15 @@ class FusedEncoder:
                 raise ValueError(f"alive must be bool or int8, got {alive.dtype}")
         if out is not None and (out.shape != x.shape or out.device != x.device):
             raise ValueError(f"out must be {tuple(x.shape)} on {x.device}")
-        # Everything the launch needs beyond x and out lives in buffers kept between calls, so a
-        # repeated call with out= given (fp32, contiguous) allocates nothing.
+        # An encoder-only launch (reference csrc/encoder.cu:1752-1764): the residual stream goes in
+        # and comes out through the tap table, the token mask replaces the board words, no heads
+        # run.  What is needed beyond x, alive and out is kept between calls, so a repeated call
+        # with out= given (fp32, contiguous) allocates nothing.
         bb = self._backbone
         if bb is None or bb["cap"] < n:
-            dev = self.device
-            bb = self._backbone = {
-                "cap": n, "boards": torch.zeros(n, T, dtype=torch.int16, device=dev),
-                "dead": torch.zeros(n, T, dtype=torch.bool, device=dev),
-                "control": torch.ones(n, dtype=torch.int16, device=dev),
-                "rep": torch.zeros(n, dtype=torch.uint8, device=dev),
-                "policy": torch.empty(n, T, N_POLICY, dtype=torch.float16, device=dev),
-                "promo": torch.empty(n, T, N_PROMO, dtype=torch.float16, device=dev),
-                "value": torch.empty(n, dtype=torch.float32, device=dev), "x": None, "y": None}
-        boards = bb["boards"][:n]
-        if alive is None:
-            boards.zero_()
-        else:
-            # a captured slot is the word 0x800; only that bit reaches the attention mask here
-            torch.logical_not(alive, out=bb["dead"][:n])
-            torch.mul(bb["dead"][:n], 0x800, out=boards)
+            bb = self._backbone = {"cap": n, "ones": torch.ones(n, T, dtype=torch.int8, device=self.device),
+                                   "x": None, "y": None}
+        alive8 = bb["ones"][:n] if alive is None else alive.contiguous()      # bool or int8: one byte, non-zero = live
         if x.dtype is torch.float32 and x.is_contiguous():
             x32 = x
         else:
@@ -871,12 +860,25 @@ class FusedEncoder:
             if bb["y"] is None or bb["y"].shape[0] < n:
                 bb["y"] = torch.empty(bb["cap"], T, d, dtype=torch.float32, device=self.device)
             y32 = bb["y"][:n]
+        for name, t_ in (("x", x), ("alive", alive), ("out", out)):
+            if t_ is not None and t_.device != self.device:
+                raise ValueError(f"{name} is on {t_.device}, the evaluator's weights are on {self.device}")
         taps = _Taps()
-        taps.x_in, taps.resid_last = x32.data_ptr(), y32.data_ptr()
+        taps.x_in, taps.resid_last, taps.alive = x32.data_ptr(), y32.data_ptr(), alive8.data_ptr()
         taps.layer_begin, taps.layer_end = 0, self.n_layers
-        # the library copies the tap table at launch; the buffers it names stay alive in the cache
-        self._call(self._args(boards, bb["control"][:n], bb["rep"][:n], None, bb["policy"][:n], bb["promo"][:n],
-                              bb["value"][:n], None, taps))
+        a = _Args()
+        a.n, a.shape = n, self._shape
+        if self.wstream is not None:
+            a.wstream, a.fparams = self.wstream.data_ptr(), self.fparams.data_ptr()
+            need = self._lib.bf_workspace_bytes(C.byref(self._shape), n)
+            if getattr(self, "workspace", None) is None or self.workspace.numel() < need:
+                self.workspace = torch.empty(need, device=self.device, dtype=torch.uint8)
+            a.workspace, a.workspace_bytes = self.workspace.data_ptr(), self.workspace.numel()
+        if self.board_wstream is not None:
+            a.board_wstream, a.board_fparams = self.board_wstream.data_ptr(), self.board_fparams.data_ptr()
+        a.kernel, a.quant, a.value_mode = self.KERNELS[self.kernel], (1 if self.fp8 else 0), self.vmode
+        a.taps = C.pointer(taps)      # the library copies the table at launch
+        self._call(a)
         if direct:
             return out
         if out is not None:

@@ -125,6 +125,12 @@ typedef struct {
     float* resid_last;  /* [B,32,d]   residual stream after the last layer run: what the
                          * reference's encoder-only call returns
                          * (brokefish/nn/cuda_impl.py:447-463) */
+    const int8_t* alive; /* [B,32] non-zero = live token.  Makes the launch encoder-only, as the
+                         * reference's encoder_forward (csrc/encoder.cu:1752-1764): x_in and
+                         * resid_last are required (they may be the same buffer: in place), the
+                         * mask of attention keys comes from here, no board words are read and no
+                         * heads run -- boards, control, rep, mask, policy, promo and value of
+                         * bf_eval_args are ignored and may be NULL */
 } bf_taps;
 
 typedef struct {
@@ -196,7 +202,7 @@ typedef struct {
  * BF_ABI_TAG before its first call and refuses a library it was not built for (a shorter
  * bf_eval_args would make the library read pointers from beyond the caller's struct).  No
  * counterpart in the reference, whose module and kernels are one compilation. */
-#define BF_ABI_VERSION 5
+#define BF_ABI_VERSION 6
 #define BF_ABI_TAG (((uint64_t)BF_ABI_VERSION << 32) | (uint64_t)sizeof(bf_eval_args))
 uint64_t bf_abi_tag(void);
 

@@ -9,7 +9,7 @@ from brokefish_amd.net import BrokefishNet
 
 def test_extension_module_loads_and_exports_the_reference_modules_functions():
     ext = hip_impl.load_extension()
-    for name in ("model_forward", "int8_q_max", "fp8_q_max", "profile_phases", "profile_phase_names", "kernel_choice"):
+    for name in ("model_forward", "encoder_forward", "int8_q_max", "fp8_q_max", "profile_phases", "profile_phase_names", "kernel_choice"):
         assert hasattr(ext, name), name
     assert ext.int8_q_max() == (127.0, 255.0) == hip_impl.int8_q_max()
     assert ext.fp8_q_max() == 8.0
@@ -71,3 +71,46 @@ def test_extension_binding_returns_the_bits_of_the_ctypes_binding_on_the_current
                              256, 8, 8, 1024, 1e-5, kernel=3, n_value=3)
     torch.cuda.synchronize()
     assert cyc.shape == (12,) and int(cyc[-1]) > 0
+
+
+@pytest.mark.gpu
+def test_encoder_forward_runs_the_stack_alone_in_place_on_every_kernel():
+    """reference csrc/encoder.cu:1752-1764: encoder_forward(y, weights, alive, ...) overwrites y with
+    the residual stream after the last layer; no board words, no heads, nothing allocated."""
+    from oracle import emulated
+    torch.manual_seed(0)
+    net = BrokefishNet().eval().randomise_layers_(seed=2)
+    sd = {k: v.detach() for k, v in net.state_dict().items()}
+    ext = hip_impl.load_extension()
+    b, c, r, _ = positions.random_positions(300, plies=100, seed=21)
+    with torch.no_grad():
+        x, alive = emulated.embed(sd, b, c, r)
+    xd, ad = x.cuda(), alive.cuda()
+    a8 = ad.to(torch.int8)                      # the mask may come as bool or as int8
+    bd, cd, rd = b.cuda(), c.cuda(), r.cuda()
+    for fp8 in (False, True):
+        kw = dict(fp8=True) if fp8 else dict(int8=True)
+        want = None
+        for kernel in ("auto", "duo", "twin", "octo", "board", "quad"):
+            mod = encoder_impl("hip")(net, kernel=kernel, **kw)
+            # what the taps of a whole-model launch record after the last layer
+            if want is None:
+                want = mod.forward_taps(bd, cd, rd, want=["resid"])["resid"][:, -1].clone()
+            quad = kernel == "quad"
+            y = xd.clone()
+            ws = torch.empty(mod._lib.bf_workspace_bytes(hip_impl.C.byref(mod._shape), 300), dtype=torch.uint8, device="cuda") if quad else None
+            count = torch.cuda.memory_stats()["allocation.all.allocated"]
+            ext.encoder_forward(y, mod.wstream if quad else mod.board_wstream, mod.fparams if quad else mod.board_fparams,
+                                a8 if kernel == "duo" else ad, 256, 8, 8, 1024, 1e-5,
+                                quant=1 if fp8 else 0, kernel=hip_impl.FusedEncoder.KERNELS[kernel], workspace=ws)
+            assert torch.cuda.memory_stats()["allocation.all.allocated"] == count
+            torch.cuda.synchronize()
+            assert torch.equal(y, want), (kernel, fp8)
+            # the class's encoder-only call is the same launch
+            assert torch.equal(mod.forward(xd, ad), want)
+    # argument errors
+    mod = encoder_impl("hip")(net, int8=True)
+    with pytest.raises(RuntimeError, match="y must be"):
+        ext.encoder_forward(xd.half(), mod.board_wstream, mod.board_fparams, ad, 256, 8, 8, 1024, 1e-5)
+    with pytest.raises(RuntimeError, match="alive must be"):
+        ext.encoder_forward(xd.clone(), mod.board_wstream, mod.board_fparams, ad[:5], 256, 8, 8, 1024, 1e-5)
