@@ -36,6 +36,7 @@ MEASURED_TRAFFIC_BYTES_E4M3 = {("base", "twin", 4096): 0.97e9}
 # with the matrix products hidden, the launch cannot be shorter than these instructions' issue time
 MEASURED_VALU_INSTS = {("base", "duo", 4096): 5.938e8, ("base", "twin", 4096): 5.513e8}
 SIMDS, CLOCK_HZ = 1024, 2.4e9
+PEAK_HBM_BPS = 8.0e12                 # MI355X HBM3E, bytes/s
 
 
 def cpu_baseline(net, batch: int, threads: int, budget_s: float = 20.0, mode: str = "int8", plies: int = 80):
@@ -96,7 +97,7 @@ def main() -> int:
                     help="base: 8 layers, width 256 (the headline metric); stress: 16 layers, width 512, "
                          "16 heads, default batch 16384")
     ap.add_argument("--kernel", choices=("auto", "quad", "board", "twin", "octo", "duo"), default="auto",
-                    help="four positions per workgroup; one position per workgroup with one (board; octo: eight wavefronts) or two (twin) workgroups per compute unit; auto: by batch size")
+                    help="four positions per workgroup (quad); one position per workgroup with one (board; octo: eight wavefronts) or two (twin) workgroups per compute unit; two positions per workgroup (duo); auto: by batch size and format")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=64)
     ap.add_argument("--no-extras", action="store_true",
@@ -107,7 +108,7 @@ def main() -> int:
                          "to calibrate FETCH_SIZE / WRITE_SIZE counter runs)")
     ap.add_argument("--phases", action="store_true",
                     help="add `phases` to the line: shader-clock ticks per wavefront and phase from the profiling "
-                         "build of the selected kernel (int8, kernels twin / octo / quad)")
+                         "build of the selected kernel")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this path runs on one GPU (positions shard with no exchange step); --gpus must be 1",
@@ -234,6 +235,7 @@ def main() -> int:
         line["stress"] = {"batch": 16384, "kernel": mdlw.kernel_choice(16384), "kernel_ms": ms, "evals_per_s": 16384 / ms * 1e3,
                           "achieved_TOPs": OPS_PER_EVAL_STRESS * 16384 / (ms * 1e-3) / 1e12,
                           "frac_int8_peak": OPS_PER_EVAL_STRESS * 16384 / (ms * 1e-3) / PEAK_INT8_OPS}
+        line["neighbours"] = neighbours(mdl8, inputs)
         del mdl8, mdlf, mdlw, wide, inputs
         line["parity"] = parity_report(net)
     if not a.no_cpu:
@@ -246,6 +248,44 @@ def main() -> int:
             line["cpu_baseline"]["fp32"] = {"value": f32["value"], "unit": "evals/s", "sample": f32["sample"]}
     print(json.dumps(line))
     return 0
+
+
+def neighbours(model, inputs):
+    """The kernels either side of the evaluator -- legal-move generation in front, the search's edge
+    expansion behind -- timed alone with events on the launch stream, with their algorithmic bytes
+    against the HBM peak (integer / byte work: 67 B of position in and 257 B of mask and check flag
+    out per position for move generation; logits, mask and position in, 96 edges out for the
+    expansion), and the chain movegen -> evaluator -> expansion on one stream."""
+    import torch
+    from brokefish_amd.hip_impl import expand_edges, movegen
+    out = []
+    for nb in (256, 4096, 65536):
+        bd, cd, rd, md = inputs[nb]
+        policy, promo, value = model.forward_full(bd, cd, rd)
+        gen = movegen(bd, cd)
+        edges = expand_edges(policy, promo, value, md, bd, cd)
+        iters = 50 if nb <= 4096 else 10
+
+        def timed(fn):
+            for _ in range(3):
+                fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            e1.synchronize()
+            return e0.elapsed_time(e1) / iters
+        t_gen = timed(lambda: movegen(bd, cd, out=gen))
+        t_exp = timed(lambda: expand_edges(policy, promo, value, md, bd, cd, out=edges))
+        t_chain = timed(lambda: model.forward_expand(bd, cd, rd, out=edges))
+        gen_bytes = nb * (64 + 2 + 256 + 1)
+        exp_bytes = nb * (2 * (32 * 64 + 32 * 4) + 4 + 256 + 64 + 2 + 96 * 4 + 4 + 4 + 4 + 2)
+        out.append({"batch": nb, "movegen_ms": t_gen, "movegen_positions_per_s": nb / t_gen * 1e3,
+                    "movegen_GBps": gen_bytes / t_gen / 1e6, "movegen_frac_hbm": gen_bytes / (t_gen * 1e-3) / PEAK_HBM_BPS,
+                    "expand_ms": t_exp, "expand_GBps": exp_bytes / t_exp / 1e6, "expand_frac_hbm": exp_bytes / (t_exp * 1e-3) / PEAK_HBM_BPS,
+                    "chain_ms": t_chain})
+    return out
 
 
 def parity_report(net):

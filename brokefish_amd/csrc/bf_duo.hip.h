@@ -173,7 +173,11 @@ __global__ __launch_bounds__(512, 1) void duo_kernel(const KArgs a) {
     // half-block `hseq` of the quarter's stream into register set `set`
     v4i frt[NSETS][4];
     auto load_half = [&](int hseq, int set) {
+#ifdef BF_EXP_SAMEBLOCK   // timing experiment: every load reads the wave's first half-block (an L1 hit)
+        const uint8_t* src = wsrc + (size_t)(hseq & 0) * HALF;
+#else
         const uint8_t* src = wsrc + (size_t)hseq * HALF;
+#endif
 #ifdef BF_EXP_NOLOAD   // timing experiment: no weight traffic
         (void)src;
 #pragma unroll

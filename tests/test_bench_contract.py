@@ -52,6 +52,10 @@ def test_one_json_line_with_roofline_and_cpu_baseline():
     assert par["bit_exact_vs_c_checker"] is True and par["masked_argmax_equal"] is True
     assert par["prior_space_vs_int8_emulation"]["max_abs"] < 1e-2 and par["prior_space_vs_int8_emulation"]["edge_set_differs"] == 0
     assert r["weight_stream"]["bytes_per_launch"] == 2048 * 6_455_296                 # two positions share a copy
+    nb = d["neighbours"]                      # move generation in front of the evaluator, edge expansion behind it
+    assert [p["batch"] for p in nb] == [256, 4096, 65536]
+    assert all(0 < p["movegen_ms"] < p["chain_ms"] and 0 < p["expand_ms"] < p["chain_ms"] for p in nb)
+    assert all(0 < p["movegen_frac_hbm"] < 1 and 0 < p["expand_frac_hbm"] < 1 for p in nb)
     assert r["weight_stream"]["achieved_TBps"] < 1.1 * r["weight_stream"]["stream_ceiling_TBps"] < 1.1 * r["weight_stream"]["l1_fill_nominal_TBps"]
 
 
