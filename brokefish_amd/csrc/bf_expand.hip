@@ -80,7 +80,12 @@ __device__ __forceinline__ unsigned ordered(float f) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-__global__ __launch_bounds__(256) void expand_kernel(const KExpand a) {
+// Three wavefronts per SIMD: left alone the compiler keeps every pass's compares alive side by side
+// in 171 registers (two wavefronts per SIMD), and a position's wavefront is a chain of dependent
+// steps that only other wavefronts can hide.  168 registers fit without a spill (30 % shorter at
+// 65536 positions); at 128 (four wavefronts) 35 registers go to scratch memory, which adds half
+// of the kernel's algorithmic bytes again as spill traffic.
+__global__ __launch_bounds__(256, 3) void expand_kernel(const KExpand a) {
     const int lane = threadIdx.x & 63;
     int b = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (b >= a.n) return;                       // no workgroup barrier below: a wave may leave
