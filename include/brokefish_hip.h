@@ -49,17 +49,20 @@ enum bf_quant {
  *   TWIN   the BOARD decomposition shaped so that two workgroups share a compute unit (each SIMD
  *          holds two wavefronts that cover each other's waits): the highest throughput
  *          (256-wide network).
- *   OCTO   the BOARD decomposition with eight wavefronts per position (two per quarter of the
- *          width, each taking half of the quarter's tiles), one workgroup per compute unit: the
- *          lowest latency per position for the 256-wide network, and the faster kernel for the
- *          512-wide one.
+ *   OCTO   eight wavefronts per position, one workgroup per compute unit: the lowest latency per
+ *          position for the 256-wide network (int8: the DUO kernel with one position per
+ *          workgroup; e4m3: the BOARD decomposition with two wavefronts per quarter of the
+ *          width), and the faster kernel for the 512-wide one (BOARD decomposition likewise).
  *   DUO    two positions per workgroup of eight wavefronts (the OCTO decomposition, every
  *          wavefront doing its share for both positions), so that a weight fragment fetched from
  *          L2 serves two positions (256-wide network, int8 and e4m3).
  * BOARD, TWIN, OCTO and DUO read the same blobs (board_wstream / board_fparams).  The 256-wide network
  * runs in int8 and e4m3 on all four; the 512-wide network in int8 on OCTO and BOARD.  Kernels that
  * carry a network and a format return bit-identical results for it, so AUTO may pick by batch
- * size. */
+ * size: OCTO up to 256 positions, above that DUO (int8) or TWIN (e4m3).  DUO runs in rounds of 512
+ * positions; when AUTO has chosen it and the last round would hold at most 256 positions, those
+ * are given to the one-position form in a second launch on the same stream (bf_kernel_choice
+ * still answers DUO). */
 enum bf_kernel {
     BF_KERNEL_AUTO = 0,
     BF_KERNEL_QUAD = 1,

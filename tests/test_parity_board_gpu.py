@@ -137,6 +137,39 @@ def test_automatic_choice_switches_kernel_by_batch_size_without_changing_results
     assert fp8.kernel_choice(1) == "octo" and fp8.kernel_choice(cut) == "octo" and fp8.kernel_choice(4096) == "twin"
 
 
+@pytest.mark.parametrize("fp16_out", [False, True])
+def test_a_small_last_round_goes_to_the_one_position_form_without_changing_results(base, fp16_out):
+    # above 512 positions the automatic choice launches the two-position kernel on the whole rounds
+    # of 512 and, when at most 256 positions remain, the one-position form on those: every output
+    # row, the skipped rows of an `active` launch and the masked argmax must be what one launch of
+    # the two-position kernel writes
+    net, sd, boards, quad, co = base
+    kw = dict(int8=True) if fp16_out else dict(int8=True, out_dtype=torch.float32)
+    auto, duo = encoder_impl("hip")(net, **kw), encoder_impl("hip")(net, kernel="duo", **kw)
+    for n in (513, 640, 768, 769, 1100, 1281):           # tails of 1, 128, 256 (split); 257, 76 + 2 rounds, 257 (not / split / not)
+        b, c, r, m = positions.random_positions(n, plies=120, seed=200 + n)
+        bd, cd, rd, md = _dev(b, c, r, m)
+        act = (torch.arange(n, device="cuda") % 5 != 0)
+        want = [t.clone() for t in duo.forward_masked(bd, cd, rd, md)]
+        got = [t.clone() for t in auto.forward_masked(bd, cd, rd, md)]
+        for x, y in zip(got, want):
+            assert torch.equal(x, y), n
+        for mod in (auto, duo):
+            for t in (mod.policy_out, mod.promo_out, mod.value_out):
+                t.fill_(3.0)
+        pa = [t.clone() for t in auto.forward_full(bd, cd, rd, active=act)]
+        pd = [t.clone() for t in duo.forward_full(bd, cd, rd, active=act)]
+        for x, y in zip(pa, pd):
+            assert torch.equal(x, y) and (x[~act] == 3.0).all(), n
+    if not fp16_out:
+        idx = np.arange(500, 640, 7)                     # rows either side of the split, against the C checker
+        b, c, r, m = positions.random_positions(640, plies=120, seed=840)
+        got = auto.forward_masked(*_dev(b, c, r, m))
+        ref = co.forward(b.numpy()[idx], c.numpy()[idx], r.numpy()[idx], mask=m.numpy()[idx])
+        assert _bits_equal(got[0][idx], ref["policy"]) and _bits_equal(got[2][idx], ref["value"])
+        assert (got[3].cpu().numpy()[idx] == ref["best"]).all()
+
+
 def test_e4m3_on_the_throughput_kernel_equals_the_four_per_workgroup_kernel(base):
     # same quantiser, same MFMA sequence per accumulator, same reduction orders: the same bits
     # (the e4m3 parity statement against the emulation is in tests/test_parity_fp8_gpu.py)
