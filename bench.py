@@ -263,8 +263,9 @@ def neighbours(model, inputs):
     """The kernels either side of the evaluator -- legal-move generation in front, the search's edge
     expansion behind -- timed alone with events on the launch stream, with their algorithmic bytes
     against the HBM peak (integer / byte work: 67 B of position in and 257 B of mask and check flag
-    out per position for move generation; logits, mask and position in, 96 edges out for the
-    expansion), and the chain movegen -> evaluator -> expansion on one stream."""
+    out per position for move generation; mask, position and the logits of the half-words that
+    hold a move in, 96 edges out for the expansion), and the chain movegen -> evaluator ->
+    expansion on one stream."""
     import torch
     from brokefish_amd.hip_impl import expand_edges, movegen
     out = []
@@ -289,7 +290,10 @@ def neighbours(model, inputs):
         t_exp = timed(lambda: expand_edges(policy, promo, value, md, bd, cd, out=edges))
         t_chain = timed(lambda: model.forward_expand(bd, cd, rd, out=edges))
         gen_bytes = nb * (64 + 2 + 256 + 1)
-        exp_bytes = nb * (2 * (32 * 64 + 32 * 4) + 4 + 256 + 64 + 2 + 96 * 4 + 4 + 4 + 4 + 2)
+        # the expansion reads a half-row of policy logits (32 fp16) only where a half-word of the mask
+        # names a move: mask, position and value in, those half-rows, 96 edges and the counters out
+        halves = int(((md & 0xFFFFFFFF) != 0).sum() + ((md >> 32) != 0).sum())
+        exp_bytes = nb * (256 + 64 + 2 + 4) + 64 * halves + nb * (96 * 4 + 4 + 4 + 4 + 2)
         out.append({"batch": nb, "movegen_ms": t_gen, "movegen_positions_per_s": nb / t_gen * 1e3,
                     "movegen_GBps": gen_bytes / t_gen / 1e6, "movegen_frac_hbm": gen_bytes / (t_gen * 1e-3) / PEAK_HBM_BPS,
                     "expand_ms": t_exp, "expand_GBps": exp_bytes / t_exp / 1e6, "expand_frac_hbm": exp_bytes / (t_exp * 1e-3) / PEAK_HBM_BPS,

@@ -10,10 +10,14 @@
 // Restates reference docs/reference/search.md:616-636 and brokefish/search/torch_impl.py:962-1033.
 //
 // One wavefront per position: lane l owns half a mask word (slot l/2, squares 32*(l%2) ..+31), so
-// lane order is canonical order and an edge's index is a prefix sum over lanes.  Nothing is
-// stored per candidate: every pass re-walks the lane's 32 squares from registers, and the
-// truncation threshold (the E-th largest log-prior) is found by bisection on the ordered bit
-// pattern of the float, so any mask is handled without a candidate buffer.
+// lane order is canonical order and an edge's index is a prefix sum over lanes.  A position has
+// some 30 legal moves over its 64 half-words, so the lanes first lay the candidates out in LDS
+// in canonical order (a lane walks only the set bits of its half-word, its logits staged in LDS)
+// and then take one to four candidates each: softmax, truncation and the stores are lane-parallel
+// over candidates, counts and ranks come from ballots.  The truncation threshold (the E-th largest
+// log-prior) is found by bisection on the ordered bit pattern of the float.  A mask with more
+// candidates than the layout holds (256; no legal position has them) is handled without it, every
+// pass walking the lanes' set bits again.
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
@@ -80,14 +84,31 @@ __device__ __forceinline__ unsigned ordered(float f) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-// Three wavefronts per SIMD: left alone the compiler keeps every pass's compares alive side by side
-// in 171 registers (two wavefronts per SIMD), and a position's wavefront is a chain of dependent
-// steps that only other wavefronts can hide.  168 registers fit without a spill (30 % shorter at
-// 65536 positions); at 128 (four wavefronts) 35 registers go to scratch memory, which adds half
-// of the kernel's algorithmic bytes again as spill traffic.
-__global__ __launch_bounds__(256, 3) void expand_kernel(const KExpand a) {
-    const int lane = threadIdx.x & 63;
-    int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+// lanes below this one whose bit is set in a ballot
+__device__ __forceinline__ int lanes_below(unsigned long long ballot) {
+    return __builtin_amdgcn_mbcnt_hi((unsigned)(ballot >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)ballot, 0));
+}
+// what one lane of this wave wrote to LDS is read by another: LDS operations of a wave are carried
+// out in program order, the fences keep the compiler from changing that order
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+constexpr int EXPAND_WAVES = 4;       // positions per workgroup
+constexpr int CAND_CAP = 256;         // candidates a wave lays out in LDS (no legal chess position has more)
+
+// FP32: the logits come as float32 (parity runs) instead of fp16 (the search contract); the staged
+// rows are then twice as large, which costs resident wavefronts, so the two are separate kernels.
+template <bool FP32>
+__global__ __launch_bounds__(64 * EXPAND_WAVES) void expand_kernel(const KExpand a) {
+    constexpr int ROW_STRIDE = (FP32 ? 128 : 64) + 16;   // bytes per lane of staged logits + a pad that spreads the banks
+    __shared__ __attribute__((aligned(16))) char row_lds[EXPAND_WAVES][64 * ROW_STRIDE];
+    __shared__ float cand_l[EXPAND_WAVES][CAND_CAP];
+    __shared__ int16_t cand_c[EXPAND_WAVES][CAND_CAP];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    int b = blockIdx.x * EXPAND_WAVES + wv;
     if (b >= a.n) return;                       // no workgroup barrier below: a wave may leave
     if (a.leaf_index) {
         if (b >= *a.leaf_count) return;
@@ -110,32 +131,28 @@ __global__ __launch_bounds__(256, 3) void expand_kernel(const KExpand a) {
     const int before = wave_exclusive(cnt, lane);
     const int total = __shfl(before + cnt, 63);
 
-    // this lane's 32 policy logits and its slot's promotion log-probabilities
-    float pol[32];
-    if (a.logits_fp32) {
-        const float* row = (const float*)a.policy + ((size_t)b * 32 + p) * 64 + 32 * half;
+    // A lane that has moves stages its 32 policy logits in LDS, where the walks below pick the
+    // ones its mask names (a lane without a move, which is most of them, loads nothing).
+    char* const myrow = row_lds[wv] + lane * ROW_STRIDE;
+    if (mh) {
+        if constexpr (FP32) {
+            const float* row = (const float*)a.policy + ((size_t)b * 32 + p) * 64 + 32 * half;
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const v4f v = *reinterpret_cast<const v4f*>(row + 4 * j);
+            for (int j = 0; j < 8; j++) *reinterpret_cast<v4f*>(myrow + 16 * j) = *reinterpret_cast<const v4f*>(row + 4 * j);
+        } else {
+            const _Float16* row = (const _Float16*)a.policy + ((size_t)b * 32 + p) * 64 + 32 * half;
 #pragma unroll
-            for (int i = 0; i < 4; i++) pol[4 * j + i] = v[i];
-        }
-    } else {
-        const _Float16* row = (const _Float16*)a.policy + ((size_t)b * 32 + p) * 64 + 32 * half;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const v8h v = *reinterpret_cast<const v8h*>(row + 8 * j);
-#pragma unroll
-            for (int i = 0; i < 8; i++) pol[8 * j + i] = (float)v[i];
+            for (int j = 0; j < 4; j++) *reinterpret_cast<v8h*>(myrow + 16 * j) = *reinterpret_cast<const v8h*>(row + 8 * j);
         }
     }
-    float lp[4];
-    {
+    // its slot's promotion log-probabilities, where a pawn reaches the last rank
+    float lp[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (pr) {
         float x[4];
 #pragma unroll
         for (int k = 0; k < 4; k++)
-            x[k] = a.logits_fp32 ? ((const float*)a.promo)[((size_t)b * 32 + p) * 4 + k]
-                                 : (float)((const _Float16*)a.promo)[((size_t)b * 32 + p) * 4 + k];
+            x[k] = FP32 ? ((const float*)a.promo)[((size_t)b * 32 + p) * 4 + k]
+                        : (float)((const _Float16*)a.promo)[((size_t)b * 32 + p) * 4 + k];
         const float mx = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
         const float s = ((__expf(x[0] - mx) + __expf(x[1] - mx)) + __expf(x[2] - mx)) + __expf(x[3] - mx);
         const float ls = __logf(s);
@@ -144,80 +161,174 @@ __global__ __launch_bounds__(256, 3) void expand_kernel(const KExpand a) {
     }
     // visit this lane's candidates in canonical order: f(log-prior, move code)
     auto each = [&](auto&& f) {
+        unsigned m = mh;
+        while (m) {
+            const int i = __builtin_ctz(m);
+            m &= m - 1;
+            const float l = FP32 ? reinterpret_cast<const float*>(myrow)[i] : (float)reinterpret_cast<const _Float16*>(myrow)[i];
+            const int mv = p * 64 + 32 * half + i;
+            if ((pr >> i) & 1u) {
 #pragma unroll
-        for (int i = 0; i < 32; i++) {
-            if ((mh >> i) & 1u) {
-                const int mv = p * 64 + 32 * half + i;
-                if ((pr >> i) & 1u) {
-#pragma unroll
-                    for (int k = 0; k < 4; k++) f(pol[i] + lp[k], mv | (k << PROMO_SHIFT));
-                } else {
-                    f(pol[i], mv);
-                }
+                for (int k = 0; k < 4; k++) f(l + lp[k], mv | (k << PROMO_SHIFT));
+            } else {
+                f(l, mv);
             }
         }
     };
-
-    float mx = -INFINITY;
-    each([&](float l, int) { mx = fmaxf(mx, l); });
-    mx = wave_max(mx);
-
-    // truncation: T = ordered pattern of the E-th largest log-prior, `need` ties at T survive
+    int16_t* const em = a.edge_move + (size_t)b * a.E;
+    _Float16* const ep = a.edge_prior + (size_t)b * a.E;
     const bool trunc = total > a.E;
-    unsigned T = 0;
-    int need = 0, tie_before = 0;
-    if (trunc) {
-        for (int bit = 31; bit >= 0; bit--) {
-            const unsigned cand = T | (1u << bit);
-            int c = 0;
-            each([&](float l, int) { c += ordered(l) >= cand; });
-            if (wave_sum(c) >= a.E) T = cand;
+    int n_edges;
+    float s_all, s_keep;
+
+    if (total <= CAND_CAP) {
+        // ---- the candidates laid out in LDS in canonical order, then one to four per lane ----------
+        float* const cl = cand_l[wv];
+        int16_t* const cc = cand_c[wv];
+        {
+            int j = before;
+            each([&](float l, int code) {
+                cl[j] = l;
+                cc[j] = (int16_t)code;
+                j++;
+            });
         }
-        int gt = 0, eq = 0;
+        wave_lds_sync();
+        constexpr int R = CAND_CAP / 64;
+        float l[R], e[R];
+        int code[R];
+        bool has[R];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int idx = lane + 64 * r;
+            has[r] = idx < total;
+            l[r] = has[r] ? cl[idx] : -INFINITY;
+            code[r] = has[r] ? cc[idx] : 0;
+            mx = fmaxf(mx, l[r]);
+        }
+        mx = wave_max(mx);
+        float sa = 0.0f;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            e[r] = has[r] ? __expf(l[r] - mx) : 0.0f;
+            sa += e[r];
+        }
+        s_all = wave_sum(sa);
+        if (!trunc) {
+            // everything survives, in place
+            n_edges = total;
+            s_keep = s_all;
+            const float inv = 1.0f / s_keep;
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                if (has[r]) {
+                    em[lane + 64 * r] = (int16_t)code[r];
+                    ep[lane + 64 * r] = (_Float16)(e[r] * inv);
+                }
+        } else {
+            // T = ordered pattern of the E-th largest log-prior, `need` ties at T survive
+            unsigned o[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) o[r] = has[r] ? ordered(l[r]) : 0u;
+            unsigned T = 0;
+#pragma clang loop unroll(disable)
+            for (int bit = 31; bit >= 0; bit--) {
+                const unsigned cand = T | (1u << bit);
+                int c = 0;
+#pragma unroll
+                for (int r = 0; r < R; r++) c += __popcll(__ballot(has[r] && o[r] >= cand));
+                if (c >= a.E) T = cand;
+            }
+            int gt = 0;
+#pragma unroll
+            for (int r = 0; r < R; r++) gt += __popcll(__ballot(has[r] && o[r] > T));
+            const int need = a.E - gt;
+            int ties = 0, kept_before = 0;
+            float sk = 0.0f;
+            bool keep[R];
+            int pos[R];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const bool eq = has[r] && o[r] == T;
+                const unsigned long long eqb = __ballot(eq);
+                keep[r] = has[r] && (o[r] > T || (eq && ties + lanes_below(eqb) < need));
+                ties += __popcll(eqb);
+                const unsigned long long kb = __ballot(keep[r]);
+                pos[r] = kept_before + lanes_below(kb);
+                kept_before += __popcll(kb);
+                sk += keep[r] ? e[r] : 0.0f;
+            }
+            n_edges = kept_before;
+            s_keep = wave_sum(sk);
+            const float inv = 1.0f / s_keep;
+#pragma unroll
+            for (int r = 0; r < R; r++)
+                if (keep[r]) {
+                    em[pos[r]] = (int16_t)code[r];
+                    ep[pos[r]] = (_Float16)(e[r] * inv);
+                }
+        }
+    } else {
+        // ---- more candidates than the layout holds (no legal position: an arbitrary mask): nothing
+        // is stored per candidate, every pass walks the lane's squares again ---------------------------
+        float mx = -INFINITY;
+        each([&](float l, int) { mx = fmaxf(mx, l); });
+        mx = wave_max(mx);
+        unsigned T = 0;
+        int need = 0, tie_before = 0;
+        if (trunc) {
+#pragma clang loop unroll(disable)
+            for (int bit = 31; bit >= 0; bit--) {
+                const unsigned cand = T | (1u << bit);
+                int c = 0;
+                each([&](float l, int) { c += ordered(l) >= cand; });
+                if (wave_sum(c) >= a.E) T = cand;
+            }
+            int gt = 0, eq = 0;
+            each([&](float l, int) {
+                const unsigned o = ordered(l);
+                gt += o > T;
+                eq += o == T;
+            });
+            need = a.E - wave_sum(gt);
+            tie_before = wave_exclusive(eq, lane);
+        }
+        // one pass: kept count of this lane, softmax denominators over all and over the survivors
+        int kept = 0, tie = tie_before;
+        float sa = 0.0f, sk = 0.0f;
         each([&](float l, int) {
-            const unsigned o = ordered(l);
-            gt += o > T;
-            eq += o == T;
+            const float e = __expf(l - mx);
+            sa += e;
+            bool keep = true;
+            if (trunc) {
+                const unsigned o = ordered(l);
+                keep = o > T || (o == T && tie < need);
+                tie += o == T;
+            }
+            if (keep) { kept++; sk += e; }
         });
-        need = a.E - wave_sum(gt);
-        tie_before = wave_exclusive(eq, lane);
+        s_all = wave_sum(sa);
+        s_keep = wave_sum(sk);
+        int pos = wave_exclusive(kept, lane);
+        n_edges = __shfl(pos + kept, 63);
+        // write the survivors in canonical order
+        const float inv = 1.0f / s_keep;
+        tie = tie_before;
+        each([&](float l, int code) {
+            bool keep = true;
+            if (trunc) {
+                const unsigned o = ordered(l);
+                keep = o > T || (o == T && tie < need);
+                tie += o == T;
+            }
+            if (keep) {
+                em[pos] = (int16_t)code;
+                ep[pos] = (_Float16)(__expf(l - mx) * inv);
+                pos++;
+            }
+        });
     }
-    // one pass: kept count of this lane, softmax denominators over all and over the survivors
-    int kept = 0, tie = tie_before;
-    float s_all = 0.0f, s_keep = 0.0f;
-    each([&](float l, int) {
-        const float e = __expf(l - mx);
-        s_all += e;
-        bool keep = true;
-        if (trunc) {
-            const unsigned o = ordered(l);
-            keep = o > T || (o == T && tie < need);
-            tie += o == T;
-        }
-        if (keep) { kept++; s_keep += e; }
-    });
-    s_all = wave_sum(s_all);
-    s_keep = wave_sum(s_keep);
-    int pos = wave_exclusive(kept, lane);
-    const int n_edges = __shfl(pos + kept, 63);
-    // write the survivors in canonical order
-    int16_t* em = a.edge_move + (size_t)b * a.E;
-    _Float16* ep = a.edge_prior + (size_t)b * a.E;
-    const float inv = 1.0f / s_keep;
-    tie = tie_before;
-    each([&](float l, int code) {
-        bool keep = true;
-        if (trunc) {
-            const unsigned o = ordered(l);
-            keep = o > T || (o == T && tie < need);
-            tie += o == T;
-        }
-        if (keep) {
-            em[pos] = (int16_t)code;
-            ep[pos] = (_Float16)(__expf(l - mx) * inv);
-            pos++;
-        }
-    });
     // unused edge slots read as no edge
     for (int i = n_edges + lane; i < a.E; i += 64) {
         em[i] = 0;
@@ -302,7 +413,9 @@ extern "C" int bf_expand(const bf_expand_args* a, void* stream) {
     k.edge_move = a->edge_move; k.edge_prior = reinterpret_cast<_Float16*>(a->edge_prior);
     k.n_edges = a->n_edges; k.count = a->count; k.dropped = a->dropped;
     k.node_value = reinterpret_cast<_Float16*>(a->node_value);
-    hipLaunchKernelGGL(expand_kernel, dim3((k.n + 3) / 4), dim3(256), 0, (hipStream_t)stream, k);
+    const dim3 grid((k.n + EXPAND_WAVES - 1) / EXPAND_WAVES), block(64 * EXPAND_WAVES);
+    if (k.logits_fp32) hipLaunchKernelGGL(expand_kernel<true>, grid, block, 0, (hipStream_t)stream, k);
+    else hipLaunchKernelGGL(expand_kernel<false>, grid, block, 0, (hipStream_t)stream, k);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         char msg[256];
