@@ -256,6 +256,28 @@ def test_kernel_truncation_ties_inactive_rows_and_dense_masks():
     assert (want["count"] >= 2048).all()
     safe = [i for i in range(4) if want["margin"][i] > 1e-5]
     _check(got, want, 4, 96, exact_rows=safe)
+    # candidate counts around the kernel's lane-parallel layout: 65..256 candidates are two to four
+    # per lane, 257 and more take the pass-per-walk path; with and without truncation, and with
+    # all-equal logits (ties cut in canonical order across the lanes' second to fourth candidates)
+    rng = np.random.default_rng(3)
+    counts = [63, 64, 65, 100, 128, 129, 200, 255, 256, 257, 300, 500]
+    dense = np.zeros((len(counts), 32), dtype=np.uint64)
+    for i, k in enumerate(counts):
+        for bit in rng.choice(2048, size=k, replace=False):
+            dense[i, bit // 64] |= np.uint64(1) << np.uint64(bit % 64)
+    dm = torch.from_numpy(dense.view(np.int64))
+    k = len(counts)
+    for E in (96, 255, 7):
+        got = expand_edges(*dev(pol[:k], pro[:k], val[:k]), dm.cuda(), b[:k].cuda(), c[:k].cuda(), E)
+        want = ox.expand(pol[:k], pro[:k], val[:k], dm.numpy(), b[:k].numpy(), c[:k].numpy(), E)
+        assert (want["count"] >= np.array(counts)).all()          # promotions only add
+        safe = [i for i in range(k) if want["margin"][i] > 1e-5]
+        assert len(safe) >= k - 1
+        _check(got, want, k, E, exact_rows=safe)
+        tie = expand_edges(*dev(zero[:k], zpro[:k], val[:k]), dm.cuda(), b[:k].cuda(), c[:k].cuda(), E)
+        wtie = ox.expand(zero[:k], zpro[:k], val[:k], dm.numpy(), b[:k].numpy(), c[:k].numpy(), E)
+        assert (tie["edge_move"].cpu().numpy() == wtie["edge_move"]).all()
+        assert (tie["n_edges"].cpu().numpy() == wtie["n_edges"]).all()
     # no legal move: zero edges, zero priors
     none = torch.zeros((4, 32), dtype=torch.int64)
     got = expand_edges(*dev(pol[:4], pro[:4], val[:4]), none.cuda(), b[:4].cuda(), c[:4].cuda(), 96)
