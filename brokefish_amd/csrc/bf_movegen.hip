@@ -5,13 +5,14 @@
 // replaying every pseudo-legal move); the CPU generator of this repository (chessgen.c, pinned by
 // the published perft counts) is its checker.
 //
-// One wavefront per position.  Every lane first builds the position's bitboards (occupancy by
-// colour, the enemy's pieces by kind) from the 32 words, broadcast lane to lane.  Lane l < 32
-// generates slot l's pseudo-legal targets with bitboard walks, and each target is tested by
-// "replaying" the move on the bitboards (occupancy, captured piece,
-// en-passant victim, castled rook) and asking whether the enemy attacks the king's square -- for
-// castling the start, crossed and landing squares, evaluated on the position after the move, as
-// the checker does.  For that step the position's moves are dealt out evenly over the 64 lanes.
+// One wavefront per position.  The position's bitboards (occupancy by colour, the enemy's pieces
+// by kind) are built once per wave on the scalar unit from the 32 words.  Lane l < 32 generates
+// slot l's pseudo-legal targets -- a slider's reach along a line is two subtractions, the other
+// pieces are shift patterns: no loop over squares -- and each target is tested by "replaying" the
+// move on the bitboards (occupancy, captured piece, en-passant victim, castled rook) and asking
+// whether the enemy attacks the king's square -- for castling the start, crossed and landing
+// squares, evaluated on the position after the move, as the checker does.  For that step the
+// position's moves are dealt out evenly over the 64 lanes.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -33,48 +34,71 @@ struct Enemy {          // the side NOT to move, after the move under test
 
 __device__ __forceinline__ u64 bit(int sq) { return 1ull << sq; }
 
-// Does `e` attack square sq, given occupancy occ?
-__device__ bool attacked(const Enemy& e, u64 occ, int sq) {
+constexpr u64 FILE_A = 0x0101010101010101ull, FILE_H = 0x8080808080808080ull;
+constexpr u64 NOT_A = ~FILE_A, NOT_H = ~FILE_H, NOT_AB = ~(FILE_A | FILE_A << 1), NOT_GH = ~(FILE_H | FILE_H >> 1);
+
+// The squares a slider on s (one bit) reaches along the line `m` (a rank, file or diagonal through
+// s, s excluded) on occupancy occ, blockers included: o - s borrows upwards through the empty
+// squares to the first blocker, so o ^ (o - s) is the ray towards the higher bits; the same on the
+// bit-reversed board is the ray towards the lower ones.  No loop, no branch.
+__device__ __forceinline__ u64 line_attacks(u64 occ, u64 m, u64 s) {
+    const u64 o = occ & m;
+    const u64 up = o - s;
+    const u64 down = __brevll(__brevll(o) - __brevll(s));
+    return (up ^ down) & m;
+}
+// the four lines through square sq (the square itself excluded)
+struct Lines { u64 rank, file, diag, anti; };
+__device__ __forceinline__ Lines lines_through(int sq) {
     const int r = sq >> 3, c = sq & 7;
+    const u64 s = bit(sq);
+    Lines l;
+    l.rank = (0xFFull << (8 * r)) ^ s;
+    l.file = (FILE_A << c) ^ s;
+    const int d = r - c;            // a1-h8 direction: 0x8040201008040201 shifted by whole ranks
+    l.diag = (d >= 0 ? 0x8040201008040201ull << (8 * d) : 0x8040201008040201ull >> (8 * -d)) ^ s;
+    const int e = r + c - 7;        // a8-h1 direction
+    l.anti = (e >= 0 ? 0x0102040810204080ull << (8 * e) : 0x0102040810204080ull >> (8 * -e)) ^ s;
+    return l;
+}
+__device__ __forceinline__ u64 rook_attacks(u64 occ, int sq) {
+    const Lines l = lines_through(sq);
+    return line_attacks(occ, l.rank, bit(sq)) | line_attacks(occ, l.file, bit(sq));
+}
+__device__ __forceinline__ u64 bishop_attacks(u64 occ, int sq) {
+    const Lines l = lines_through(sq);
+    return line_attacks(occ, l.diag, bit(sq)) | line_attacks(occ, l.anti, bit(sq));
+}
+__device__ __forceinline__ u64 knight_pattern(u64 s) {
+    return ((s << 17) & NOT_A) | ((s << 10) & NOT_AB) | ((s >> 6) & NOT_AB) | ((s >> 15) & NOT_A) |
+           ((s << 15) & NOT_H) | ((s << 6) & NOT_GH) | ((s >> 10) & NOT_GH) | ((s >> 17) & NOT_H);
+}
+__device__ __forceinline__ u64 king_pattern(u64 s) {
+    const u64 row = s | ((s << 1) & NOT_A) | ((s >> 1) & NOT_H);
+    return (row | row << 8 | row >> 8) ^ s;
+}
+
+// Does `e` attack square sq, given occupancy occ?  Looked at from the square: a rook placed there
+// sees the enemy's orthogonal sliders exactly when they see it, and so for the other kinds.
+__device__ __forceinline__ bool attacked(const Enemy& e, u64 occ, int sq) {
+    const u64 s = bit(sq);
     // a white pawn on (r-1, c+-1) attacks (r, c); a black one from (r+1, c+-1)
-    const int pr = e.black ? r + 1 : r - 1;
-    if (pr >= 0 && pr < 8) {
-        if (c > 0 && (e.pawns & bit(pr * 8 + c - 1))) return true;
-        if (c < 7 && (e.pawns & bit(pr * 8 + c + 1))) return true;
-    }
-    const int kn[8][2] = {{1, 2}, {2, 1}, {2, -1}, {1, -2}, {-1, -2}, {-2, -1}, {-2, 1}, {-1, 2}};
-    const int kg[8][2] = {{1, 0}, {1, 1}, {0, 1}, {-1, 1}, {-1, 0}, {-1, -1}, {0, -1}, {1, -1}};
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-        int rr = r + kn[i][0], cc = c + kn[i][1];
-        if (rr >= 0 && rr < 8 && cc >= 0 && cc < 8 && (e.knights & bit(rr * 8 + cc))) return true;
-        rr = r + kg[i][0]; cc = c + kg[i][1];
-        if (rr >= 0 && rr < 8 && cc >= 0 && cc < 8 && (e.king & bit(rr * 8 + cc))) return true;
-    }
-    const int ray[8][2] = {{1, 0}, {-1, 0}, {0, 1}, {0, -1}, {1, 1}, {1, -1}, {-1, 1}, {-1, -1}};
-#pragma unroll
-    for (int d = 0; d < 8; d++) {
-        int rr = r + ray[d][0], cc = c + ray[d][1];
-        while (rr >= 0 && rr < 8 && cc >= 0 && cc < 8) {
-            const u64 b = bit(rr * 8 + cc);
-            if (occ & b) {
-                if ((d < 4 ? e.orth : e.diag) & b) return true;
-                break;
-            }
-            rr += ray[d][0]; cc += ray[d][1];
-        }
-    }
-    return false;
+    const u64 pawn_from = e.black ? (((s << 7) & NOT_H) | ((s << 9) & NOT_A)) : (((s >> 7) & NOT_A) | ((s >> 9) & NOT_H));
+    const u64 hit = (pawn_from & e.pawns) | (knight_pattern(s) & e.knights) | (king_pattern(s) & e.king) |
+                    (rook_attacks(occ, sq) & e.orth) | (bishop_attacks(occ, sq) & e.diag);
+    return hit != 0;
 }
 
 __global__ __launch_bounds__(256) void movegen_kernel(const uint16_t* boards, const int16_t* control, int n,
                                                       u64* mask, uint8_t* in_check) {
     const int lane = threadIdx.x & 63;
-    const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+    // the position and the side to move are the same for the whole wave: said so, the bitboard
+    // construction below runs on the scalar unit
+    const int b = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
     if (b >= n) return;                                 // no workgroup barrier below
     const int slot = lane & 31, part = lane >> 5;
     const unsigned w = boards[(size_t)b * 32 + slot];
-    const bool black = control[b] < 0;
+    const bool black = __builtin_amdgcn_readfirstlane((int)control[b]) < 0;
 
     // bitboards, computed by every lane from the words of all 32 slots
     u64 own = 0, opp = 0, ep_pawns = 0;
@@ -84,7 +108,7 @@ __global__ __launch_bounds__(256) void movegen_kernel(const uint16_t* boards, co
     const unsigned rookw = (black ? COLOR : 0u) | (ROOK << 6);
 #pragma unroll
     for (int s = 0; s < 32; s++) {
-        const unsigned v = (unsigned)__shfl((int)w, s);
+        const unsigned v = (unsigned)__builtin_amdgcn_readlane((int)w, s);   // wave-uniform: the loop runs on the scalar unit
         rook_short |= v == (rookw | (row + 7));
         rook_long |= v == (rookw | row);
         if (v & CAPTURED) continue;
@@ -102,7 +126,7 @@ __global__ __launch_bounds__(256) void movegen_kernel(const uint16_t* boards, co
         }
     }
     const u64 occ = own | opp;
-    const int ksq = __shfl((int)w, black ? 31 : 15) & 63;
+    const int ksq = (black ? __builtin_amdgcn_readlane((int)w, 31) : __builtin_amdgcn_readlane((int)w, 15)) & 63;
     if (lane == 0 && in_check) in_check[b] = attacked(e, occ, ksq) ? 1 : 0;
 
     // pseudo-legal targets of this slot
@@ -127,34 +151,18 @@ __global__ __launch_bounds__(256) void movegen_kernel(const uint16_t* boards, co
                     if (r == (black ? 3 : 4) && (ep_pawns & bit(r * 8 + cc))) ps |= bit(r1 * 8 + cc);
                 }
             }
-        } else if (t == KNIGHT || t == KING) {
-            const int kn[8][2] = {{1, 2}, {2, 1}, {2, -1}, {1, -2}, {-1, -2}, {-2, -1}, {-2, 1}, {-1, 2}};
-            const int kg[8][2] = {{1, 0}, {1, 1}, {0, 1}, {-1, 1}, {-1, 0}, {-1, -1}, {0, -1}, {1, -1}};
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const int rr = r + (t == KNIGHT ? kn[i][0] : kg[i][0]), cc = c + (t == KNIGHT ? kn[i][1] : kg[i][1]);
-                if (rr < 0 || rr > 7 || cc < 0 || cc > 7) continue;
-                if (!(own & bit(rr * 8 + cc))) ps |= bit(rr * 8 + cc);
-            }
-            if (t == KING && !(w & SPECIAL)) {
+        } else if (t == KNIGHT) {
+            ps = knight_pattern(bit(sq)) & ~own;
+        } else if (t == KING) {
+            ps = king_pattern(bit(sq)) & ~own;
+            if (!(w & SPECIAL)) {
                 if (rook_short && !(occ & (bit(row + 5) | bit(row + 6)))) ps |= bit(row + 6);
                 if (rook_long && !(occ & (bit(row + 1) | bit(row + 2) | bit(row + 3)))) ps |= bit(row + 2);
             }
         } else if (t == BISHOP || t == ROOK || t == QUEEN) {
-            const int ray[8][2] = {{1, 0}, {-1, 0}, {0, 1}, {0, -1}, {1, 1}, {1, -1}, {-1, 1}, {-1, -1}};
-            const int d0 = (t == BISHOP) ? 4 : 0, d1 = (t == ROOK) ? 4 : 8;
-            for (int d = d0; d < d1; d++) {
-                int rr = r + ray[d][0], cc = c + ray[d][1];
-                while (rr >= 0 && rr < 8 && cc >= 0 && cc < 8) {
-                    const u64 sb = bit(rr * 8 + cc);
-                    if (occ & sb) {
-                        if (opp & sb) ps |= sb;
-                        break;
-                    }
-                    ps |= sb;
-                    rr += ray[d][0]; cc += ray[d][1];
-                }
-            }
+            if (t != BISHOP) ps |= rook_attacks(occ, sq);
+            if (t != ROOK) ps |= bishop_attacks(occ, sq);
+            ps &= ~own;
         }
     }
 
