@@ -1,6 +1,6 @@
 """The device chain (move generation -> evaluator -> edge expansion) under HIP graph capture.
 
-Small launches are launch-bound (a 64-position evaluation is 0.16 ms of kernel time), so a search
+Small launches are latency-bound (a 64-position evaluation is 0.12 ms of kernel time), so a search
 would capture the chain once and replay it.  None of the three entry points allocates, waits on
 the host or clears memory with a memset node, so the chain can be captured as it is.  Each replay
 is checked against the eager chain on the same inputs, with eager work and synchronisations
