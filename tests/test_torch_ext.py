@@ -114,3 +114,44 @@ def test_encoder_forward_runs_the_stack_alone_in_place_on_every_kernel():
         ext.encoder_forward(xd.half(), mod.board_wstream, mod.board_fparams, ad, 256, 8, 8, 1024, 1e-5)
     with pytest.raises(RuntimeError, match="alive must be"):
         ext.encoder_forward(xd.clone(), mod.board_wstream, mod.board_fparams, ad[:5], 256, 8, 8, 1024, 1e-5)
+
+
+@pytest.mark.gpu
+def test_two_evaluators_on_two_streams_and_two_host_threads_do_not_disturb_each_other():
+    """The library keeps no state between calls but the per-thread error text: launches from two
+    host threads on two streams (default priority), overlapping on the GPU, return what each
+    evaluator returns alone.  Kernels that need no scratch buffer are used (the four-per-workgroup
+    kernel's workspace belongs to its evaluator object, so that one is safe as well and is included)."""
+    import threading
+    torch.manual_seed(0)
+    nets = [BrokefishNet().eval().randomise_layers_(seed=s) for s in (3, 4)]
+    inputs = [tuple(t.cuda() for t in positions.random_positions(n, plies=120, seed=50 + i)) for i, n in enumerate((777, 200))]
+    for kernel in ("auto", "quad"):
+        models = [encoder_impl("hip")(net, int8=True, kernel=kernel) for net in nets]
+        alone = [[t.clone() for t in m.forward_masked(*x)] for m, x in zip(models, inputs)]
+        torch.cuda.synchronize()
+        streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+        results, errors = [None, None], []
+
+        def work(i):
+            try:
+                with torch.cuda.stream(streams[i]):
+                    out = None
+                    for _ in range(30):                      # long enough for the two loops to overlap
+                        out = models[i].forward_masked(*inputs[i])
+                    results[i] = [t.clone() for t in out]
+                streams[i].synchronize()
+            except Exception as e:                            # surfaced in the main thread below
+                errors.append(e)
+        for s in streams:
+            s.wait_stream(torch.cuda.current_stream())
+        threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join(timeout=120)
+        assert not errors and all(not th.is_alive() for th in threads), errors
+        torch.cuda.synchronize()
+        for got, want in zip(results, alone):
+            for g, w in zip(got, want):
+                assert torch.equal(g, w), kernel
