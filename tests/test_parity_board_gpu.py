@@ -573,3 +573,28 @@ def test_set_profile_accumulates_over_calls_until_reset_like_the_references_swit
     assert model.read_profile()[1] == w2
     model.reset_profile()
     assert model.read_profile()[1] == 0
+
+
+def test_two_hundred_thousand_positions_agree_bit_for_bit_across_the_kernels(base):
+    # size-independent property at the sweep's largest launches: the kernels are the same function
+    # (two positions per workgroup, one per workgroup with two workgroups per unit, four per
+    # workgroup, and the automatic choice with its split last round), in int8 and in e4m3, on
+    # launches whose sizes are multiples of nothing; a sample goes against the C checker
+    net, sd, boards, quad, co = base
+    hip = encoder_impl("hip")
+    mods = {k: hip(net, int8=True, out_dtype=torch.float32, kernel=k) for k in ("duo", "twin", "auto")}
+    f8 = {k: hip(net, fp8=True, out_dtype=torch.float32, kernel=k) for k in ("duo", "twin")}
+    for seed, n in ((0, 65536), (1, 65536 - 771), (2, 65536 + 130)):
+        b, c, r, m = positions.random_positions(n, plies=200, seed=3000 + seed)
+        dev = _dev(b, c, r, m)
+        ref = [t.clone() for t in mods["duo"].forward_masked(*dev)]
+        for other in (mods["twin"], mods["auto"], quad):
+            for g, w in zip(other.forward_masked(*dev), ref):
+                assert torch.equal(g, w), seed
+        e = [t.clone() for t in f8["duo"].forward_masked(*dev)]
+        for g, w in zip(f8["twin"].forward_masked(*dev), e):
+            assert torch.equal(g, w), seed
+        idx = np.arange(seed, n, 1999)
+        want = co.forward(b.numpy()[idx], c.numpy()[idx], r.numpy()[idx], mask=m.numpy()[idx])
+        assert _bits_equal(ref[0][idx], want["policy"]) and _bits_equal(ref[1][idx], want["promo"])
+        assert _bits_equal(ref[2][idx], want["value"]) and (ref[3].cpu().numpy()[idx] == want["best"]).all()
