@@ -124,7 +124,19 @@ def build_torch_ext() -> str:
     return TORCH_EXT
 
 
+C_DRIVER = os.path.join(os.path.dirname(HERE), "tests", "abi", "c_driver")
+
+
+def build_c_driver() -> str:
+    """tests/abi/c_driver: a host program over the C-ABI and the HIP runtime alone (no PyTorch), for
+    the GPU test that runs the library without Python.  Host code only; the library must be built."""
+    _run([hipcc_path(), "-O2", "-std=c++17", "-I", INCLUDE, C_DRIVER + ".cpp", "-o", C_DRIVER,
+          "-L", HERE, "-lbrokefish_hip", "-Wl,-rpath," + HERE])
+    return C_DRIVER
+
+
 def build_all(verbose: bool = False) -> None:
     build_chessgen()
     build_hip(verbose)
     build_torch_ext()
+    build_c_driver()
