@@ -16,6 +16,25 @@ def test_more_than_one_gpu_is_refused_with_a_message():
     assert run.returncode != 0 and "one GPU" in run.stderr and run.stdout.strip() == ""
 
 
+def test_the_traffic_and_instruction_tables_quote_the_committed_profile_summaries():
+    # `roofline.traffic` and `valu_floor_ms` are not measured inside the bench process: they are the
+    # counter results of the profile summaries.  A table entry that no summary holds has gone stale.
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    text = {f: open(os.path.join(ROOT, "profiles", f)).read() for f in os.listdir(os.path.join(ROOT, "profiles"))}
+    where = {("base", "duo", 4096): "duo_kernel_int8_batch4096.md", ("base", "twin", 4096): "board_kernel_twin_int8_batch4096.md",
+             ("base", "quad", 4096): "eval_kernel_quad_int8_batch4096.md", ("base", "octo", 256): "duo_kernel_solo_int8_batch256.md",
+             ("stress", "octo", 16384): "board_kernel_octo_512_int8_batch16384.md"}
+    for key, name in where.items():
+        assert key in bench.MEASURED_TRAFFIC_BYTES and name in text, key
+    assert "0.445e9" in text["duo_kernel_int8_batch4096.md"] and bench.MEASURED_TRAFFIC_BYTES[("base", "duo", 4096)] == 0.445e9
+    assert "0.78e9" in text["board_kernel_twin_int8_batch4096.md"] and bench.MEASURED_TRAFFIC_BYTES[("base", "twin", 4096)] == 0.78e9
+    assert "5.938e8" in text["duo_kernel_int8_batch4096.md"] and bench.MEASURED_VALU_INSTS[("base", "duo", 4096)] == 5.938e8
+    assert "5.513e8" in text["board_kernel_twin_int8_batch4096.md"] and bench.MEASURED_VALU_INSTS[("base", "twin", 4096)] == 5.513e8
+
+
 @pytest.mark.gpu
 def test_one_json_line_with_roofline_and_cpu_baseline():
     run = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "5", "--warmup", "2", "--cpu-batch", "16"],
