@@ -12,6 +12,11 @@
 // workgroup barrier.  The arithmetic is that of the other kernels operation for operation, so
 // the results are bit-identical to theirs.
 //
+// NPOS = 1 is the same kernel with one position per workgroup: the latency form for launches of
+// at most one workgroup per compute unit (each wavefront one tile of the width, every product
+// issued under the previous product's epilogue, and the workgroups of an XCD warming the L2
+// with the next layer's weights one layer ahead).
+//
 // LDS map (bytes): [xch: 3 slots x 2 positions x 8 waves x 64 floats] [hid: the quantised hidden
 // row, 32 KiB per position] [act: the quantised row of the width, 8 KiB per position] [par: one
 // copy of each quarter's side parameters, shared by its two wavefronts and both positions]
@@ -21,7 +26,8 @@
 
 #include "bf_board.hip.h"
 
-// register sets of the weight prefetch (one set = half a block; SETS - 1 half-blocks in flight)
+// register sets of the weight prefetch (one set = half a block; a set is refilled the moment its
+// half-block has been consumed, so all of them are in flight or full between products)
 #ifndef BF_DUO_SETS
 #define BF_DUO_SETS 3
 #endif
