@@ -21,22 +21,21 @@ HIP_LIB = os.path.join(HERE, "libbrokefish_hip.so")
 CHESSGEN_LIB = os.path.join(HERE, "libbf_chessgen.so")
 TORCH_EXT = os.path.join(HERE, "_bf_torch.so")
 
-HIP_SOURCES = ["bf_host.hip", "bf_expand.hip", "bf_movegen.hip", "bf_probe.hip", "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip",
-               "bf_variant_prod_fp8.hip", "bf_variant_taps_fp8.hip",
-               "bf_variant_board256.hip", "bf_variant_board256_taps.hip",
-               "bf_variant_board512.hip", "bf_variant_board512_taps.hip",
-               "bf_variant_twin256.hip", "bf_variant_twin256_taps.hip",
-               "bf_variant_twin256_fp8.hip", "bf_variant_twin256_fp8_taps.hip",
-               "bf_variant_board256_fp8.hip", "bf_variant_board256_fp8_taps.hip",
-               "bf_variant_octo512.hip", "bf_variant_octo512_taps.hip",
-               "bf_variant_octo256_fp8.hip", "bf_variant_octo256_fp8_taps.hip",
-               "bf_variant_duo256.hip", "bf_variant_duo256_taps.hip",
-               "bf_variant_duo256_fp8.hip", "bf_variant_duo256_fp8_taps.hip",
-               "bf_variant_twin256_prof.hip", "bf_variant_duo256_prof.hip",
-               "bf_variant_solo256.hip", "bf_variant_solo256_taps.hip", "bf_variant_solo256_prof.hip", "bf_variant_octo512_prof.hip",
-               "bf_variant_board256_prof.hip", "bf_variant_board512_prof.hip", "bf_variant_board256_fp8_prof.hip",
-               "bf_variant_twin256_fp8_prof.hip", "bf_variant_octo256_fp8_prof.hip", "bf_variant_duo256_fp8_prof.hip",
-               "bf_variant_prof_fp8.hip"]
+# the four-positions-per-workgroup kernels take minutes each to compile (the e4m3 ones five): they
+# go first so that the pool's last minutes are not spent waiting for one of them alone
+HIP_SOURCES = ["bf_variant_prod_fp8.hip", "bf_variant_taps_fp8.hip", "bf_variant_prof_fp8.hip",
+               "bf_variant_prod.hip", "bf_variant_taps.hip", "bf_variant_prof.hip",
+               "bf_variant_board512.hip", "bf_variant_board512_taps.hip", "bf_variant_board512_prof.hip",
+               "bf_host.hip", "bf_expand.hip", "bf_movegen.hip", "bf_probe.hip",
+               "bf_variant_board256.hip", "bf_variant_board256_taps.hip", "bf_variant_board256_prof.hip",
+               "bf_variant_twin256.hip", "bf_variant_twin256_taps.hip", "bf_variant_twin256_prof.hip",
+               "bf_variant_twin256_fp8.hip", "bf_variant_twin256_fp8_taps.hip", "bf_variant_twin256_fp8_prof.hip",
+               "bf_variant_board256_fp8.hip", "bf_variant_board256_fp8_taps.hip", "bf_variant_board256_fp8_prof.hip",
+               "bf_variant_octo512.hip", "bf_variant_octo512_taps.hip", "bf_variant_octo512_prof.hip",
+               "bf_variant_octo256_fp8.hip", "bf_variant_octo256_fp8_taps.hip", "bf_variant_octo256_fp8_prof.hip",
+               "bf_variant_duo256.hip", "bf_variant_duo256_taps.hip", "bf_variant_duo256_prof.hip",
+               "bf_variant_duo256_fp8.hip", "bf_variant_duo256_fp8_taps.hip", "bf_variant_duo256_fp8_prof.hip",
+               "bf_variant_solo256.hip", "bf_variant_solo256_taps.hip", "bf_variant_solo256_prof.hip"]
 # -ffp-contract=off: the kernel's fp32 arithmetic is specified operation by operation
 # (fused multiply-adds are written explicitly), so the compiler must not fuse on its own.
 # The packed-fp32 feature is disabled so no v_pk_*_f32 instructions are generated.
